@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused Adam step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[3], the one the metric is quoted on): a single rank's OSS shard of a
+13B model -- one contiguous buffer of 1.63e9 parameters, MEMORY_EFFICIENT_MIXED_PRECISION (fp16
+params and grads, fp32 m/v, grads scaled by 1024).  A "step" is one ``Adam.step()`` over that shard
+with everything resident in HBM.  Prints ONE JSON line; the same shard stepped in MIXED_PRECISION
+(fp32 master + fp16 grads + fp16 copy-out, 28 B/param) is reported under "also".
+
+"roofline" prices the dominant kernel against 8 TB/s of HBM: algorithmic bytes per launch (22 B per
+parameter in this mode: reads p16,g16,m32,v32, writes p16,m32,v32) over the kernel's average duration
+measured with HIP events on the launch stream.  "cpu_baseline" times the same math as in-place torch
+CPU ops on the host cores for a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBS = 8000.0
+BYTES_PER_PARAM = {"FULL_PRECISION": 28, "MIXED_PRECISION": 28, "MEMORY_EFFICIENT_MIXED_PRECISION": 22, "PURE_FP16": 14}
+SHARD_NUMEL = 1_630_000_000
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--numel", type=int, default=SHARD_NUMEL, help="parameters in the flat shard")
+    ap.add_argument("--mode", default="MEMORY_EFFICIENT_MIXED_PRECISION", choices=list(BYTES_PER_PARAM))
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary MIXED_PRECISION measurement")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-numel", type=int, default=1 << 26, help="sample size of the CPU baseline")
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (chunk_elems, wg_per_cu, nontemporal, unroll)")
+    return ap.parse_args()
+
+
+def make_shard(torch, precision_name, numel, device):
+    """Flat parameter + gradient of the mode's dtypes, generated on the device (synthetic)."""
+    gen = torch.Generator(device=device).manual_seed(4000)
+    scale = 1024.0
+    if precision_name == "FULL_PRECISION":
+        p = torch.empty(numel, device=device, dtype=torch.float32).normal_(0, 0.02, generator=gen)
+        g = torch.empty(numel, device=device, dtype=torch.float32).normal_(0, 1e-3, generator=gen)
+        scale = 1.0
+    else:
+        p = torch.empty(numel, device=device, dtype=torch.float16).normal_(0, 0.02, generator=gen)
+        g = torch.empty(numel, device=device, dtype=torch.float16).normal_(0, 1e-3 * scale, generator=gen)
+    p.requires_grad_()
+    p.grad = g
+    return p, scale
+
+
+def time_steps(torch, opt, scale, steps, warmup):
+    """W untimed steps, then K steps between synchronisations; wall time and HIP-event time (events sit
+    on torch's current stream, which is the stream the optimizer hands to the library)."""
+    for _ in range(warmup):
+        opt.step(scale=scale)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        opt.step(scale=scale)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) / 1e3
+
+
+def measure_gpu(torch, precision_name, numel, steps, warmup, device):
+    from fairscale_amd.optim import Adam, Precision
+
+    p, scale = make_shard(torch, precision_name, numel, device)
+    opt = Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, precision=getattr(Precision, precision_name))
+    wall, dev_s = time_steps(torch, opt, scale, steps, warmup)
+    plan = next(iter(opt._plans.values())).info()
+    assert torch.isfinite(p.detach()[:4096].float()).all()
+    bpp = BYTES_PER_PARAM[precision_name]
+    kernel_s = dev_s / steps  # one launch per step: plan["n_launches"] == 1
+    out = {
+        "params_per_s": numel * steps / wall,
+        "ms_per_step": wall / steps * 1e3,
+        "kernel_ms": kernel_s * 1e3,
+        "bytes_per_param": bpp,
+        "achieved_gbs": numel * bpp / kernel_s / 1e9,
+        "plan": {k: plan[k] for k in ("n_launches", "grid", "block", "chunk_elems", "total_chunks", "n_vector_tensors")},
+    }
+    del opt, p
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_cpu(torch, precision_name, numel, budget_s=20.0):
+    """The same math as in-place torch CPU ops on `numel` parameters; stops after ~budget_s."""
+    from oracle import adam_oracle as O
+    from oracle.adam_torch_cpu import step_torch_cpu
+
+    mode = {"FULL_PRECISION": O.FULL_PRECISION, "MIXED_PRECISION": O.MIXED_PRECISION,
+            "MEMORY_EFFICIENT_MIXED_PRECISION": O.MEMORY_EFFICIENT_MIXED_PRECISION, "PURE_FP16": O.PURE_FP16}[precision_name]
+    pd = torch.float32 if mode in (O.FULL_PRECISION, O.MIXED_PRECISION) else torch.float16
+    gd = torch.float32 if mode == O.FULL_PRECISION else torch.float16
+    sd = torch.float16 if mode == O.PURE_FP16 else torch.float32
+    gen = torch.Generator().manual_seed(4000)
+    scale = 1.0 if mode == O.FULL_PRECISION else 1024.0
+    p = (torch.randn(numel, generator=gen) * 0.02).to(pd)
+    g = (torch.randn(numel, generator=gen) * (1e-3 * scale)).to(gd)
+    m, v = torch.zeros(numel, dtype=sd), torch.zeros(numel, dtype=sd)
+    pc = torch.zeros(numel, dtype=torch.float16) if mode == O.MIXED_PRECISION else None
+    kw = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, grad_scale=scale, optim_scale=65536.0 if mode == O.PURE_FP16 else 1.0)
+    step_torch_cpu(mode, p, m, v, g, pc, step=1, **kw)  # warm-up
+    done, t0 = 0, time.perf_counter()
+    while True:
+        step_torch_cpu(mode, p, m, v, g, pc, step=2 + done, **kw)
+        done += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or done >= 50:
+            break
+    return {"value": numel * done / el, "unit": "params/s", "cores": int(torch.get_num_threads()), "kind": "port",
+            "sample": f"{done} steps of the same {precision_name} math (in-place torch CPU ops, oracle/adam_torch_cpu.py) on a flat {numel}-parameter buffer, {el:.1f} s"}
+
+
+def load_traffic(workload_key):
+    """HBM bytes per launch from the committed counter summary, if there is one for this workload."""
+    path = os.path.join(REPO, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as fh:
+            return json.load(fh).get(workload_key, {}).get("traffic_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: the Adam step of one rank's shard needs no communication, so "
+              f"--gpus {args.gpus} is not supported (every rank would run this same kernel on its own shard).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from fairscale_amd import _cabi
+
+    for item in args.opt:
+        name, value = item.split("=")
+        _cabi.set_option(name, int(value))
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    main_res = measure_gpu(torch, args.mode, args.numel, args.steps, args.warmup, device)
+    also = {}
+    if not args.no_also and args.mode != "MIXED_PRECISION":
+        r = measure_gpu(torch, "MIXED_PRECISION", args.numel, args.steps, args.warmup, device)
+        also["MIXED_PRECISION"] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
+                                   "achieved_gbs": r["achieved_gbs"], "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
+    cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
+
+    workload = f"flat_shard_{args.numel}_{args.mode}"
+    line = {
+        "metric": "params updated/sec + HBM GB/s (% of peak), 1.6B-param shard, mixed precision",
+        "value": main_res["params_per_s"],
+        "unit": "params/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 arithmetic; fp16 params+grads, fp32 m/v" if args.mode == "MEMORY_EFFICIENT_MIXED_PRECISION" else "f32 arithmetic",
+        "data": "synthetic",
+        "config": {"workload": workload, "numel": args.numel, "precision": args.mode, "tensors": 1, "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
+                   "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
+                   "options": {k: _cabi.get_option(k) for k in ("chunk_elems", "wg_per_cu", "nontemporal", "unroll")}},
+        "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": load_traffic(workload),
+                     "kernel": "fsadam_kernel", "kernel_ms": main_res["kernel_ms"], "bytes_per_param": main_res["bytes_per_param"]},
+        "cpu_baseline": cpu,
+        "also": also,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,50 @@
+"""Compiles fsadam.hip into libfsadam.so next to this file (hipcc, gfx950 only).
+
+Usage: ``python -m fairscale_amd.csrc.build`` or ``build_library()``.  The library is kept in-tree so
+that a process which loads it shows it among its mapped files.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REPO = os.path.dirname(os.path.dirname(HERE))
+SOURCE = os.path.join(HERE, "fsadam.hip")
+LIBRARY = os.path.join(HERE, "libfsadam.so")
+INCLUDE = os.path.join(REPO, "include")
+
+# -ffp-contract=off: multiplies and adds stay separate, as the update equations are written.
+# No -ffast-math: division and square root stay correctly rounded, isfinite logic stays meaningful.
+# packed fp32 arithmetic is switched off for the device code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
+
+
+def build_library(verbose: bool = False) -> str:
+    """Always recompiles; returns the path of the shared library."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", INCLUDE, "-o", LIBRARY + ".tmp", SOURCE]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    noise = "is not a recognized feature for this target"  # the host pass does not know the device feature
+    log = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
+    os.replace(LIBRARY + ".tmp", LIBRARY)
+    if verbose and log.strip():
+        print(log, file=sys.stderr)
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

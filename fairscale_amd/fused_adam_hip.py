@@ -1,0 +1,177 @@
+"""Python face of the native step: same call as ``fairscale.fused_adam_cuda.adam``.
+
+Reference: pybind module ``fairscale/clib/fused_adam_cuda/fused_adam_cuda.cpp:4-8``, dispatcher
+``fused_adam_cuda_kernel.cu:137-265``, list validation ``multi_tensor_apply.cuh:49-67``.  Here the
+tensor lists are turned into rows of plain pointers and handed to ``libfsadam.so`` through ctypes;
+the kernels run on torch's current HIP stream and the call does not wait for them.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _cabi
+
+__all__ = ["adam", "TensorListPlan", "mode_of_lists", "rows_of_lists"]
+
+_ROW_WORDS = ctypes.sizeof(_cabi.FsAdamTensor) // 8
+assert _ROW_WORDS == 6, "FsAdamTensor is five pointers and one int64"
+
+
+def mode_of_lists(tensor_lists: Sequence[Sequence[torch.Tensor]]) -> int:
+    """dtype dispatch of fused_adam_cuda_kernel.cu:165-263 (looks at the first tensor of each list)."""
+    depth = len(tensor_lists)
+    if depth not in (4, 5):
+        raise RuntimeError("tensor_lists.size() != depth")  # multi_tensor_apply.cuh:49
+    if len(tensor_lists[0]) == 0:
+        raise RuntimeError("tensor_lists[0].size() is not > 0")  # multi_tensor_apply.cuh:51
+    p, m, v, g = (tensor_lists[d][0].dtype for d in range(4))
+    if m != v:
+        raise RuntimeError("exp_avg and exp_avg_sq must have the same dtype")  # kernel.cu:167
+    if depth == 5:
+        if p != torch.float32 or g != torch.float16 or tensor_lists[4][0].dtype != torch.float16 or m != torch.float32:
+            raise RuntimeError("mixed precision expects fp32 params/state with fp16 grads and fp16 output params")  # kernel.cu:174-176
+        return _cabi.MIXED_PRECISION
+    if p != g:
+        raise RuntimeError("params and grads must have the same dtype")  # kernel.cu:196
+    if p == torch.float32:
+        if m != torch.float32:
+            raise RuntimeError("Optimizer state must be of type float for float parameters")  # kernel.cu:199
+        return _cabi.FULL_PRECISION
+    if p == torch.float16:
+        if m == torch.float32:
+            return _cabi.MEMORY_EFFICIENT_MIXED_PRECISION
+        if m == torch.float16:
+            return _cabi.PURE_FP16
+        raise RuntimeError("Optimizer state must be of type float or half")  # kernel.cu:258
+    raise RuntimeError("Parameters must be of type float or half")  # kernel.cu:261
+
+
+_MODE_DTYPES = {
+    _cabi.FULL_PRECISION: (torch.float32, torch.float32, torch.float32, torch.float32),
+    _cabi.MIXED_PRECISION: (torch.float32, torch.float32, torch.float32, torch.float16, torch.float16),
+    _cabi.MEMORY_EFFICIENT_MIXED_PRECISION: (torch.float16, torch.float32, torch.float32, torch.float16),
+    _cabi.PURE_FP16: (torch.float16, torch.float16, torch.float16, torch.float16),
+}
+
+
+def validate_lists(tensor_lists: Sequence[Sequence[torch.Tensor]], mode: int) -> torch.device:
+    """The checks of multi_tensor_apply.cuh:49-67, plus dtype/device uniformity (the kernels index raw
+    memory, so what the reference leaves to asserts is enforced here).  Returns the lists' device."""
+    dtypes = _MODE_DTYPES[mode]
+    if len(tensor_lists) != len(dtypes):
+        raise RuntimeError("tensor_lists.size() != depth")
+    len0 = len(tensor_lists[0])
+    if len0 == 0:
+        raise RuntimeError("tensor_lists[0].size() is not > 0")
+    device = tensor_lists[0][0].device
+    for lst, dtype in zip(tensor_lists, dtypes):
+        if len(lst) != len0:
+            raise RuntimeError("Size mismatch among tensor lists")
+        for t, t0 in zip(lst, tensor_lists[0]):
+            if not t.is_contiguous():
+                raise RuntimeError("A tensor was not contiguous.")
+            if not t.is_cuda:
+                raise RuntimeError("A tensor was not cuda.")
+            if t.numel() != t0.numel():
+                raise RuntimeError("Size mismatch")
+            if t.dtype != dtype:
+                raise RuntimeError(f"A tensor has dtype {t.dtype}, the list needs {dtype}.")
+            if t.device != device:
+                raise RuntimeError("Tensors of one call must live on one device.")
+    return device
+
+
+def rows_of_lists(tensor_lists: Sequence[Sequence[torch.Tensor]]) -> np.ndarray:
+    """(n, 6) int64: p, m, v, g, p_copy pointers and numel -- the memory layout of FsAdamTensor[n]."""
+    n = len(tensor_lists[0])
+    rows = np.zeros((n, _ROW_WORDS), dtype=np.int64)
+    for d, lst in enumerate(tensor_lists):
+        rows[:, d] = [t.data_ptr() for t in lst]
+    rows[:, 5] = [t.numel() for t in tensor_lists[0]]
+    return rows
+
+
+def _rows_ptr(rows: np.ndarray):
+    return rows.ctypes.data_as(ctypes.POINTER(_cabi.FsAdamTensor))
+
+
+def _stream_handle(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def adam(chunk_size: int, noop_flag: Optional[torch.Tensor], tensor_lists: List[List[torch.Tensor]], lr: float,
+         beta1: float, beta2: float, eps: float, grad_scale: float, optim_scale: float, found_inf: torch.Tensor,
+         step: int, mode: int, bias_correction: int, decay: float) -> None:
+    """Drop-in for ``fairscale.fused_adam_cuda.adam`` (fused_adam_cuda.cpp:4-8; call site adam.py:261-276).
+
+    ``tensor_lists`` is ``[p, m, v, g]`` or ``[p32, m, v, g16, p16_out]``; ``mode`` is the eps mode
+    (0 inside the square root, 1 outside).  ``chunk_size`` and ``noop_flag`` are accepted for
+    signature compatibility and ignored: chunking is internal, and the reference kernel never reads
+    ``noop_flag`` (fused_adam_cuda_kernel.cu:26).  ``found_inf`` is a float32[1] device tensor that is
+    set to 1.0 when a stored fp16 ``m``/``v`` is non-finite (PURE_FP16 only) and never cleared.
+    """
+    precision = mode_of_lists(tensor_lists)
+    device = validate_lists(tensor_lists, precision)
+    if found_inf is None or found_inf.dtype != torch.float32 or not found_inf.is_cuda or found_inf.numel() < 1:
+        raise RuntimeError("found_inf must be a float32 device tensor with one element")
+    if found_inf.device != device:
+        raise RuntimeError("found_inf must live on the tensors' device")
+    rows = rows_of_lists(tensor_lists)
+    L = _cabi.lib()
+    with torch.cuda.device(device):
+        _cabi.check(L.fsadam_step(_rows_ptr(rows), rows.shape[0], precision, lr, beta1, beta2, eps, grad_scale,
+                                  optim_scale, decay, int(step), int(mode), int(bias_correction),
+                                  found_inf.data_ptr(), _stream_handle(device)))
+
+
+class TensorListPlan:
+    """A tensor list whose device-side table is kept between steps (fsadam_plan_* in include/fsadam.h).
+
+    The optimizer holds one per (param group, device).  ``step`` re-reads every pointer, and only
+    when one moved (or the list changed length) is the list validated again and its table re-sent.
+    """
+
+    def __init__(self, precision: int, device: torch.device):
+        self.precision = precision
+        self.device = device
+        self._rows: Optional[np.ndarray] = None
+        self._handle = ctypes.c_void_p()
+        _cabi.check(_cabi.lib().fsadam_plan_create(precision, ctypes.byref(self._handle)))
+
+    def close(self) -> None:
+        if self._handle:
+            try:
+                _cabi.lib().fsadam_plan_destroy(self._handle)
+            finally:
+                self._handle = ctypes.c_void_p()
+
+    def __del__(self):  # pragma: no cover - interpreter shutdown order is not ours to test
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def info(self) -> dict:
+        out = _cabi.FsAdamPlanInfo()
+        _cabi.check(_cabi.lib().fsadam_plan_info(self._handle, ctypes.byref(out)))
+        return out.as_dict()
+
+    def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,
+             grad_scale: float, optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int,
+             bias_correction: int, decay: float) -> None:
+        L = _cabi.lib()
+        rows = rows_of_lists(tensor_lists)
+        with torch.cuda.device(self.device):
+            stream = _stream_handle(self.device)
+            if self._rows is None or rows.shape != self._rows.shape or not np.array_equal(rows, self._rows):
+                if validate_lists(tensor_lists, self.precision) != self.device:
+                    raise RuntimeError("tensor list moved to another device")
+                _cabi.check(L.fsadam_plan_set_tensors(self._handle, _rows_ptr(rows), rows.shape[0], stream))
+                self._rows = rows
+            flag = found_inf.data_ptr() if found_inf is not None else None
+            _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, grad_scale, optim_scale, decay,
+                                           int(step), int(eps_mode), int(bias_correction), flag, stream))

@@ -1,0 +1,295 @@
+"""``Adam`` / ``Precision``: the interface of ``fairscale/optim/adam.py`` over the gfx950 kernels.
+
+Same constructor, attributes, ``state_dict`` keys, exceptions and optimizer-state-scale behaviour as
+the reference class (``fairscale/optim/adam.py:42-297``); the native call it makes per (param group,
+device) goes to ``libfsadam.so`` instead of ``fairscale.fused_adam_cuda``.
+
+Deliberate differences, all supersets of the reference behaviour:
+
+* ``step(closure=None, *, scale=1.0)``: the gradient scale the kernel divides by is reachable through
+  the class (the reference hard-codes 1.0, adam.py:238, although its docstring lists ``scale``).
+* ``lr``/``eps``/``betas``/``weight_decay`` are range-checked (``ValueError``), which is what
+  ``tests/optim/test_adam.py:357-370`` expects.
+* The device flag is only allocated, cleared and read back in PURE_FP16: the other three modes cannot
+  raise it (fused_adam_cuda_kernel.cu:94-105 is the only writer), so they step without a host sync.
+  The scale bookkeeping they do every step (adam.py:289-295) is kept.
+* After an overflow m and v are zeroed in place rather than re-allocated (adam.py:285-288), and
+  parameters that never had a gradient keep an empty state instead of a half-initialised one.
+* ``load_state_dict`` keeps fp32 ``exp_avg``/``exp_avg_sq`` exact for fp16 parameters (the reference
+  round-trips them through fp16, adam.py:176-182).
+"""
+from __future__ import annotations
+
+from enum import Enum, auto
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from .. import _cabi
+from ..fused_adam_hip import TensorListPlan
+
+_cabi.lib()  # loading the kernels is part of importing the optimizer: no library, no Adam
+
+__all__ = ["Adam", "Precision"]
+
+
+class Precision(Enum):
+    """Where parameters, gradients and optimizer state live (adam.py:19-23)."""
+
+    FULL_PRECISION = auto()
+    MIXED_PRECISION = auto()
+    MEMORY_EFFICIENT_MIXED_PRECISION = auto()
+    PURE_FP16 = auto()
+
+
+_NATIVE_MODE = {
+    Precision.FULL_PRECISION: _cabi.FULL_PRECISION,
+    Precision.MIXED_PRECISION: _cabi.MIXED_PRECISION,
+    Precision.MEMORY_EFFICIENT_MIXED_PRECISION: _cabi.MEMORY_EFFICIENT_MIXED_PRECISION,
+    Precision.PURE_FP16: _cabi.PURE_FP16,
+}
+
+_MAX_OPTIM_SCALE = 2 ** 16
+
+
+class _DeviceBatch:
+    """The tensor lists of one param group on one device, in the order the native call wants them."""
+
+    __slots__ = ("lists",)
+
+    def __init__(self, depth: int):
+        self.lists: List[List[torch.Tensor]] = [[] for _ in range(depth)]
+
+    def add(self, tensors: Tuple[torch.Tensor, ...]) -> None:
+        for lst, t in zip(self.lists, tensors):
+            lst.append(t)
+
+
+class Adam(torch.optim.Optimizer):
+    """Fused Adam on MI355X. GPU-only.
+
+    Arguments (as ``fairscale.optim.Adam``, adam.py:76-88):
+        params: iterable of parameters (a flat list; the precision is read off the first one).
+        lr: learning rate (default 1e-3).
+        bias_correction: apply the ``sqrt(1-beta2^t)/(1-beta1^t)`` factor to the step (default True).
+        betas: running-average coefficients (default (0.9, 0.999)).
+        eps: denominator term (default 1e-8); it is NOT rescaled by the bias correction.
+        eps_inside_sqrt: ``sqrt(v + eps)`` instead of ``sqrt(v) + eps`` (default False).
+        weight_decay: ``p -= step_size * weight_decay * p`` (default 0).
+        max_grad_norm: stored in ``defaults`` and unused, as in the reference.
+        amsgrad: not supported (``RuntimeError``).
+        precision: a ``Precision``; inferred from the first parameter when None (fp32 ->
+            FULL_PRECISION, otherwise MIXED_PRECISION).
+    """
+
+    state: dict
+    defaults: dict
+
+    def __init__(
+        self,
+        params: Any,
+        lr: Optional[float] = 1e-3,
+        bias_correction: Optional[bool] = True,
+        betas: Optional[Tuple[float, float]] = (0.9, 0.999),
+        eps: Optional[float] = 1e-8,
+        eps_inside_sqrt: Optional[bool] = False,
+        weight_decay: Optional[float] = 0.0,
+        max_grad_norm: Optional[float] = 0.0,
+        amsgrad: Optional[bool] = False,
+        precision: Optional[Precision] = None,
+    ):
+        parameters: List[Any] = list(params)
+        first_dtype = parameters[0].dtype
+        if precision is None:  # adam.py:92-95
+            precision = Precision.FULL_PRECISION if first_dtype == torch.float32 else Precision.MIXED_PRECISION
+        self.precision = precision
+        if precision is not Precision.FULL_PRECISION:  # adam.py:97-98
+            assert first_dtype == torch.float16
+
+        pure_fp16 = precision is Precision.PURE_FP16
+        self.optim_type = torch.float16 if pure_fp16 else torch.float32  # adam.py:100
+        self._optim_scale = float(_MAX_OPTIM_SCALE) if pure_fp16 else 1.0  # adam.py:101
+        self._steps_since_optim_scale_change = 0
+        self._optim_scale_update_freq = 2000  # GradScaler's default growth interval (adam.py:103)
+        # kept for interface parity; the native step never reads it (fused_adam_cuda_kernel.cu:26)
+        self._overflow_buf = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+        if amsgrad:
+            raise RuntimeError("FusedAdam does not support the AMSGrad variant.")
+        if lr is not None and not 0.0 <= lr:
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if eps is not None and not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon value: {eps}")
+        if betas is not None:
+            for k, beta in enumerate(betas):
+                if not 0.0 <= beta < 1.0:
+                    raise ValueError(f"Invalid beta parameter at index {k}: {beta}")
+        if weight_decay is not None and not 0.0 <= weight_decay:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+
+        super().__init__(
+            parameters,
+            dict(lr=lr, bias_correction=bias_correction, betas=betas, eps=eps, weight_decay=weight_decay,
+                 max_grad_norm=max_grad_norm),
+        )
+        self.eps_mode = 0 if eps_inside_sqrt else 1  # adam.py:117
+
+        self.fp32_param_groups: List[Any] = []
+        if self.mixed_precision:
+            self._build_fp32_params(parameters)
+
+        self._plans: Dict[Tuple[int, torch.device], TensorListPlan] = {}
+        self._flags: Dict[torch.device, torch.Tensor] = {}
+
+    # ------------------------------------------------------------------ interface of the reference
+
+    def _build_fp32_params(self, params: Any) -> None:
+        """fp32 master copies of fp16 parameters, one group (adam.py:123-153)."""
+        masters = []
+        for p in params:
+            master = torch.nn.Parameter(p.data.float()).to(p.device)
+            master.grad = torch.zeros_like(master.data)
+            masters.append(master)
+        group: Dict[str, Any] = {"params": masters}
+        for name, default in self.defaults.items():
+            group.setdefault(name, default)
+        self.fp32_param_groups = [group]
+
+    @property
+    def supports_memory_efficient_fp16(self) -> bool:
+        return True
+
+    @property
+    def _step_supports_amp_scaling(self) -> bool:
+        return False
+
+    @property
+    def mixed_precision(self) -> bool:
+        return self.precision is Precision.MIXED_PRECISION
+
+    def state_dict(self) -> Dict[str, Any]:
+        out = super().state_dict()
+        out["optim_scale"] = self._optim_scale  # adam.py:169
+        return out
+
+    def load_state_dict(self, state_dict: Dict[str, Any]) -> None:
+        super().load_state_dict(state_dict)
+        self._optim_scale = state_dict["optim_scale"]  # adam.py:174
+        # torch casts floating state to the parameter dtype; take m and v from the saved tensors instead
+        # so that fp32 state of fp16 parameters is restored bit for bit.
+        saved_ids = [pid for g in state_dict["param_groups"] for pid in g["params"]]
+        live = [p for g in self.param_groups for p in g["params"]]
+        saved_state = state_dict["state"]
+        for pid, p in zip(saved_ids, live):
+            if pid not in saved_state or p not in self.state:
+                continue
+            for key in ("exp_avg", "exp_avg_sq"):
+                if key in saved_state[pid]:
+                    src = saved_state[pid][key]
+                    self.state[p][key] = src.detach().to(device=p.device, dtype=self.optim_type, copy=True)
+        self._plans_invalidate()
+
+    # ------------------------------------------------------------------ the step
+
+    def _plans_invalidate(self) -> None:
+        for plan in self.__dict__.get("_plans", {}).values():
+            plan.close()
+        self._plans = {}
+
+    def _flag_for(self, device: torch.device) -> torch.Tensor:
+        flag = self._flags.get(device)
+        if flag is None:
+            flag = torch.zeros(1, dtype=torch.float32, device=device)
+            self._flags[device] = flag
+        return flag
+
+    def step(self, closure: Optional[Callable[[], float]] = None, *, scale: float = 1.0) -> Optional[float]:
+        """One optimization step (adam.py:184-297).
+
+        Arguments:
+            closure: re-evaluates the model and returns the loss.
+            scale: gradients are divided by this inside the kernel (loss-scale folded into the step).
+        """
+        loss = closure() if closure is not None else None
+        self.__dict__.setdefault("_plans", {})  # absent after unpickling
+        self.__dict__.setdefault("_flags", {})
+        native_mode = _NATIVE_MODE[self.precision]
+        mixed = self.mixed_precision
+        watch_overflow = self.precision is Precision.PURE_FP16
+
+        for gi, group in enumerate(self.param_groups):
+            batches: Dict[torch.device, _DeviceBatch] = {}
+            beta1, beta2 = group["betas"]
+            step_no = None
+            for pj, p in enumerate(group["params"]):
+                if p.grad is None:
+                    continue
+                grad = p.grad.data
+                if grad.is_sparse:
+                    raise RuntimeError("FusedAdam does not support sparse gradients, please consider SparseAdam instead")
+                state = self.state[p]
+                if len(state) == 0:  # adam.py:223-228
+                    state["step"] = 0
+                    state["exp_avg"] = torch.zeros_like(p, dtype=self.optim_type)
+                    state["exp_avg_sq"] = torch.zeros_like(p, dtype=self.optim_type)
+                state["step"] += 1
+                step_no = state["step"]  # the call uses the last parameter's counter (adam.py:272)
+                batch = batches.get(p.device)
+                if batch is None:
+                    batch = batches[p.device] = _DeviceBatch(5 if mixed else 4)
+                if mixed:
+                    master = self.fp32_param_groups[gi]["params"][pj]
+                    batch.add((master.data, state["exp_avg"], state["exp_avg_sq"], grad, p.data))
+                else:
+                    batch.add((p.data, state["exp_avg"], state["exp_avg_sq"], grad))
+
+            if not batches:
+                # adam.py:256 indexes the first device of an empty dict
+                raise IndexError("list index out of range")
+
+            flags: List[torch.Tensor] = []
+            for device, batch in batches.items():
+                flag = None
+                if watch_overflow:
+                    flag = self._flag_for(device)
+                    flag.zero_()
+                    flags.append(flag)
+                plan = self._plans.get((gi, device))
+                if plan is None:
+                    plan = self._plans[(gi, device)] = TensorListPlan(native_mode, device)
+                plan.step(batch.lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
+                          step_no, self.eps_mode, 1 if group["bias_correction"] else 0, group["weight_decay"])
+
+            overflowed = bool(sum(f.item() for f in flags)) if flags else False  # adam.py:278
+            if overflowed:
+                self._steps_since_optim_scale_change = 0
+                self._optim_scale /= 2
+                if self._optim_scale < 1.0:
+                    raise RuntimeError("Optimizer state scale < 1. This may mean that gradients are exploding")
+                self._zero_all_state()
+            else:
+                self._steps_since_optim_scale_change += 1
+
+            if self._steps_since_optim_scale_change == self._optim_scale_update_freq:  # adam.py:292-295
+                self._steps_since_optim_scale_change = 0
+                if self._optim_scale < _MAX_OPTIM_SCALE:
+                    self._optim_scale *= 2
+
+        return loss
+
+    def _zero_all_state(self) -> None:
+        """m = v = 0 for every parameter of every group (adam.py:285-288)."""
+        stale: List[torch.Tensor] = []
+        for group in self.param_groups:
+            for p in group["params"]:
+                state = self.state.get(p)
+                if not state:
+                    continue
+                for key in ("exp_avg", "exp_avg_sq"):
+                    t = state.get(key)
+                    if t is not None and t.dtype == self.optim_type and t.shape == p.shape and t.device == p.device:
+                        stale.append(t)
+                    else:
+                        state[key] = torch.zeros_like(p, dtype=self.optim_type)
+        if stale:
+            torch._foreach_zero_(stale)
