@@ -41,7 +41,10 @@ def parse_args():
     ap.add_argument("--no-also", action="store_true", help="skip the secondary MIXED_PRECISION measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-numel", type=int, default=1 << 26, help="sample size of the CPU baseline")
-    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (chunk_elems, wg_per_cu, nontemporal, unroll)")
+    ap.add_argument("--calib-copy-bytes", type=int, default=0,
+                    help="first run the library's plain copy kernel over this many bytes three times (a dispatch of known "
+                         "traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (block, groups, lds_throttle, xcd_remap)")
     return ap.parse_args()
 
 
@@ -94,14 +97,14 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
         "kernel_ms": kernel_s * 1e3,
         "bytes_per_param": bpp,
         "achieved_gbs": numel * bpp / kernel_s / 1e9,
-        "plan": {k: plan[k] for k in ("n_launches", "grid", "block", "chunk_elems", "total_chunks", "n_vector_tensors")},
+        "plan": {k: plan[k] for k in ("n_launches", "grid", "block", "tile_elems", "n_descriptors", "lds_throttle", "n_vector_tensors")},
     }
     del opt, p
     torch.cuda.empty_cache()
     return out
 
 
-def measure_cpu(torch, precision_name, numel, budget_s=20.0):
+def measure_cpu(torch, precision_name, numel, budget_s=15.0):
     """The same math as in-place torch CPU ops on `numel` parameters; stops after ~budget_s."""
     from oracle import adam_oracle as O
     from oracle.adam_torch_cpu import step_torch_cpu
@@ -124,7 +127,7 @@ def measure_cpu(torch, precision_name, numel, budget_s=20.0):
         step_torch_cpu(mode, p, m, v, g, pc, step=2 + done, **kw)
         done += 1
         el = time.perf_counter() - t0
-        if el > budget_s or done >= 50:
+        if el > budget_s or done >= 2000:
             break
     return {"value": numel * done / el, "unit": "params/s", "cores": int(torch.get_num_threads()), "kind": "port",
             "sample": f"{done} steps of the same {precision_name} math (in-place torch CPU ops, oracle/adam_torch_cpu.py) on a flat {numel}-parameter buffer, {el:.1f} s"}
@@ -159,6 +162,16 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.calib_copy_bytes > 0:
+        n = args.calib_copy_bytes // 16 * 16
+        src = torch.zeros(n, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            _cabi.check(_cabi.lib().fsadam_calib_copy(dst.data_ptr(), src.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     main_res = measure_gpu(torch, args.mode, args.numel, args.steps, args.warmup, device)
     also = {}
     if not args.no_also and args.mode != "MIXED_PRECISION":
@@ -183,10 +196,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": workload, "numel": args.numel, "precision": args.mode, "tensors": 1, "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
                    "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
-                   "options": {k: _cabi.get_option(k) for k in ("chunk_elems", "wg_per_cu", "nontemporal", "unroll")}},
+                   "options": {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap")}},
         "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": load_traffic(workload),
-                     "kernel": "fsadam_kernel", "kernel_ms": main_res["kernel_ms"], "bytes_per_param": main_res["bytes_per_param"]},
+                     "kernel": "fsadam_tiles", "kernel_ms": main_res["kernel_ms"], "bytes_per_param": main_res["bytes_per_param"]},
         "cpu_baseline": cpu,
         "also": also,
     }

@@ -32,24 +32,25 @@ class FsAdamTensor(ctypes.Structure):
     ]
 
 
-class FsAdamPlanInfo(ctypes.Structure):
-    _fields_ = [
-        ("mode", ctypes.c_int32),
-        ("device", ctypes.c_int32),
-        ("n_tensors", ctypes.c_int64),
-        ("total_elems", ctypes.c_int64),
-        ("total_chunks", ctypes.c_int64),
-        ("chunk_elems", ctypes.c_int64),
-        ("n_vector_tensors", ctypes.c_int64),
-        ("n_scalar_tensors", ctypes.c_int64),
-        ("n_launches", ctypes.c_int64),
-        ("grid", ctypes.c_int64),
-        ("block", ctypes.c_int64),
-        ("uploads", ctypes.c_int64),
-    ]
-
+class _Int64Fields(ctypes.Structure):
     def as_dict(self) -> dict:
         return {name: int(getattr(self, name)) for name, _ in self._fields_}
+
+
+class FsAdamPlanInfo(_Int64Fields):
+    _fields_ = [("mode", ctypes.c_int32), ("device", ctypes.c_int32)] + [
+        (name, ctypes.c_int64)
+        for name in ("n_tensors", "total_elems", "tile_elems", "large_chunk_elems", "n_descriptors", "n_vector_tensors",
+                     "n_scalar_tensors", "n_launches", "grid", "block", "lds_throttle", "uploads")
+    ]
+
+
+class FsAdamLayout(_Int64Fields):
+    _fields_ = [
+        (name, ctypes.c_int64)
+        for name in ("tile_elems", "large_chunk_elems", "n_large_tensors", "n_small_tensors", "n_empty_tensors",
+                     "n_large_descriptors", "n_small_descriptors", "grid_large", "grid_small")
+    ]
 
 
 # name -> (restype, argtypes); one entry per function include/fsadam.h declares
@@ -67,7 +68,7 @@ SIGNATURES = {
     "fsadam_plan_step": (_i32, [_vp] + _SCALARS + [_vp, _vp]),
     "fsadam_plan_info": (_i32, [_vp, ctypes.POINTER(FsAdamPlanInfo)]),
     "fsadam_plan_destroy": (_i32, [_vp]),
-    "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, _i64, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint8)]),
+    "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),
     "fsadam_clear_cache": (_i32, []),
     "fsadam_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
 }

@@ -5,23 +5,32 @@
 //                                                                dtype dispatch :172-256)
 //   fairscale/clib/fused_adam_cuda/multi_tensor_apply.cuh      (tensor-list launcher :40-130)
 //
-// Design, in one paragraph.  The path is elementwise and HBM-bound (14-28 bytes per element, a few
-// dozen flops), so there is no MFMA here; the job is to keep every HBM channel busy.  The tensor list
-// lives in a device-resident table (one 64-byte row per tensor) that is uploaded once and reused
-// every step; an exclusive prefix sum of per-tensor chunk counts turns "work item c" into (tensor,
-// chunk) by a binary search that every workgroup runs out of LDS, so ONE launch covers any number
-// of tensors (the reference needs one launch per 36 tensors / 320 chunks because its table travels
-// by value in the kernel arguments).  Workgroups of four wave64s walk the work items grid-stride;
-// inside an item every lane moves 128-bit vectors (two per fp32 stream, one per fp16 stream in the
-// half-precision modes) with several independent loads in flight before the first use, does the
-// update in fp32 registers, and writes p, m, v (and the fp16 copy of p) back with 128-bit stores.
-// Tensors with a stream that is not 16-byte aligned, and the ragged last few elements of a tensor,
-// go through an element-wise path with the same arithmetic.
+// Design.  The path is elementwise and HBM-bound (14-28 bytes per element against a few dozen
+// flops), so there is no MFMA here; what decides the speed is how the memory system is driven.
+// Measured on this part, a streaming kernel is fastest when
+//   * every workgroup is "one-shot": it handles one small tile (a few KiB per stream) and exits, so
+//     that the hardware dispatcher hands out tiles in address order and the set of DRAM pages in
+//     use at any moment stays small (grid-stride loops let workgroups drift apart and lose ~20 %);
+//   * only 6-12 waves are resident per compute unit: enough bytes in flight to cover the latency,
+//     few enough that the active address window stays tight.  Residency is capped by giving each
+//     workgroup a block of LDS it never touches (LDS is the one launch-time resource that bounds
+//     residency without costing registers or bandwidth);
+//   * every load/store instruction of a wave covers one contiguous span (lane i next to lane i+1),
+//     128 bits per lane for fp32 streams and 64 or 128 bits per lane for fp16 streams, all with
+//     the non-temporal hint (nothing is re-read).
+// The tensor list becomes a device-resident table of 64-byte chunk descriptors (five pointers
+// already advanced to the chunk, element count, alignment flag), uploaded once and reused every
+// step.  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
+// tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles, small tensors get
+// one descriptor per tile in a second launch, so ONE or TWO launches cover any number of tensors
+// (the reference needs a launch per 36 tensors / 320 chunks because its table travels by value in
+// the kernel arguments).  Tiles that are ragged (end of a tensor) or belong to a tensor with a
+// misaligned stream take an element-wise path with the same arithmetic.
 //
 // Arithmetic is IEEE float32 exactly as written in the reference source: separate multiplies and
 // adds (compiled with -ffp-contract=off), correctly rounded division and square root (hipcc's
-// default for fp32), round-to-nearest-even conversions to fp16.  Dividing by a power-of-two scale is
-// done as a multiplication by its exact reciprocal, which gives the same bits.
+// default for fp32), round-to-nearest-even conversions to fp16.  Dividing by a power-of-two scale
+// is done as a multiplication by its exact reciprocal, which gives the same bits.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -42,38 +51,33 @@ namespace {
 // shared host/device definitions
 // --------------------------------------------------------------------------------------------
 
-constexpr int kBlock = 256;          // 4 wave64 per workgroup
-constexpr int kWindow = 8192;        // tensors whose chunk prefix one launch stages in LDS (32 KiB + 4)
-constexpr int kChunkQuantum = 2048;  // chunk_elems granularity: keeps chunk bases 16-byte aligned in every dtype
+constexpr int64_t kLargeThreshold = 131072;   // tensors with at least this many elements share descriptors
+constexpr int64_t kMinLargeChunk = 65536;     // elements per shared descriptor, lower bound
+constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room)
 
-struct alignas(16) TensorRow {  // 64 bytes
+struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points at the chunk's first element
     void* p;
     void* m;
     void* v;
     const void* g;
     void* p_copy;
-    int64_t numel;
-    uint32_t vector_ok;  // every stream 16-byte aligned
-    uint32_t pad;
+    uint32_t n;          // elements in this chunk (<= chunk size of its launch)
+    uint32_t vector_ok;  // every stream aligned for the vector path
+    uint64_t pad;
 };
-static_assert(sizeof(TensorRow) == 64, "table row must stay 64 bytes");
-
-enum : int { kGradScalePow2 = 1, kOptimScalePow2 = 2 };
+static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");
 
 struct StepScalars {
     float b1, b2, one_minus_b1, one_minus_b2;
     float eps, decay, step_size;
     float grad_scale, inv_grad_scale;
     float optim_scale, inv_optim_scale;
-    int eps_mode;  // 0: sqrt(v+eps), 1: sqrt(v)+eps
-    int flags;     // kGradScalePow2 | kOptimScalePow2
+    int eps_mode;     // 0: sqrt(v+eps), 1: sqrt(v)+eps
+    int fast_scales;  // every scale the mode divides by is a power of two with an exact reciprocal
 };
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-// Pointers read out of the tensor table would otherwise be generic (flat_* instructions, which also
-// tie up the LDS counter); these live in global memory, so say so.
+// Pointers read out of the descriptor table would otherwise be generic (flat_* instructions, which
+// also tie up the LDS counter); these live in global memory, so say so.
 #define FS_GLOBAL __attribute__((address_space(1)))
 template <typename T>
 using gptr = FS_GLOBAL T*;
@@ -84,115 +88,81 @@ template <>
 struct ModeTraits<FSADAM_FULL_PRECISION> {
     using P = float; using G = float; using S = float;
     static constexpr bool kCopy = false, kScaled = false;
-    static constexpr int kVec = 4;
+    static constexpr int kElems = 4;  // elements per lane per group: 16 bytes of the widest stream
 };
 template <>
 struct ModeTraits<FSADAM_MIXED_PRECISION> {
     using P = float; using G = _Float16; using S = float;
     static constexpr bool kCopy = true, kScaled = false;
-    static constexpr int kVec = 8;
+    static constexpr int kElems = 4;
 };
 template <>
 struct ModeTraits<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION> {
     using P = _Float16; using G = _Float16; using S = float;
     static constexpr bool kCopy = false, kScaled = false;
-    static constexpr int kVec = 8;
+    static constexpr int kElems = 4;
 };
 template <>
 struct ModeTraits<FSADAM_PURE_FP16> {
     using P = _Float16; using G = _Float16; using S = _Float16;
     static constexpr bool kCopy = false, kScaled = true;
-    static constexpr int kVec = 8;
+    static constexpr int kElems = 8;
 };
+
+constexpr int mode_elems(int mode) { return mode == FSADAM_PURE_FP16 ? 8 : 4; }
 
 // --------------------------------------------------------------------------------------------
 // device code
 // --------------------------------------------------------------------------------------------
 
-// N consecutive elements of T held as raw 16-byte quads until they are needed.
-template <typename T, int N>
-struct Packet {
-    static constexpr int kQuads = N * (int)sizeof(T) / 16;
-    static_assert(kQuads >= 1 && kQuads * 16 == N * (int)sizeof(T), "packet must be whole 16-byte quads");
-    f32x4 q[kQuads];
+template <typename T, int E>
+struct VecOf {
+    typedef T type __attribute__((ext_vector_type(E)));
 };
 
-template <typename T, int N, bool NT>
-__device__ __forceinline__ Packet<T, N> load_packet(gptr<const T> ptr) {
-    Packet<T, N> r;
-    gptr<const f32x4> src = reinterpret_cast<gptr<const f32x4>>(ptr);
-#pragma unroll
-    for (int k = 0; k < Packet<T, N>::kQuads; ++k) {
-        if (NT)
-            r.q[k] = __builtin_nontemporal_load(src + k);
-        else
-            r.q[k] = src[k];
-    }
-    return r;
+// E consecutive elements of one stream, one instruction, non-temporal.
+template <typename T, int E>
+__device__ __forceinline__ typename VecOf<T, E>::type load_vec(gptr<const T> ptr) {
+    using V = typename VecOf<T, E>::type;
+    return __builtin_nontemporal_load(reinterpret_cast<gptr<const V>>(ptr));
+}
+template <typename T, int E>
+__device__ __forceinline__ void store_vec(gptr<T> ptr, typename VecOf<T, E>::type value) {
+    using V = typename VecOf<T, E>::type;
+    __builtin_nontemporal_store(value, reinterpret_cast<gptr<V>>(ptr));
 }
 
-template <typename T, int N, bool NT>
-__device__ __forceinline__ void store_packet(gptr<T> ptr, const Packet<T, N>& r) {
-    gptr<f32x4> dst = reinterpret_cast<gptr<f32x4>>(ptr);
-#pragma unroll
-    for (int k = 0; k < Packet<T, N>::kQuads; ++k) {
-        if (NT)
-            __builtin_nontemporal_store(r.q[k], dst + k);
-        else
-            dst[k] = r.q[k];
-    }
+// Two packed halves in one 32-bit word: non-zero when either is +-inf or NaN (exponent field all
+// ones).  Adding 0x0400 to an all-ones exponent field carries into the sign position; any smaller
+// field does not, and the low half cannot carry into the high one.  The test is kept in integer
+// arithmetic on whole words on purpose: written as per-element comparisons OR-ed into a bool, the
+// compiler's vectorised form only looked at the first element of each packet.
+__device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w) {
+    return ((w & 0x7c007c00u) + 0x04000400u) & 0x80008000u;
 }
 
-template <int N>
-__device__ __forceinline__ void unpack(const Packet<float, N>& r, float (&out)[N]) {
+template <int E>
+__device__ __forceinline__ uint32_t nonfinite_in(typename VecOf<_Float16, E>::type h) {
+    static_assert(E == 4 || E == 8, "whole 32-bit words only");
+    typedef uint32_t words_t __attribute__((ext_vector_type(E / 2)));
+    const words_t w = __builtin_bit_cast(words_t, h);
+    uint32_t bad = 0;
 #pragma unroll
-    for (int k = 0; k < N; ++k) out[k] = r.q[k / 4][k % 4];
-}
-template <int N>
-__device__ __forceinline__ void unpack(const Packet<_Float16, N>& r, float (&out)[N]) {
-#pragma unroll
-    for (int k = 0; k < N / 8; ++k) {
-        const f16x8 h = __builtin_bit_cast(f16x8, r.q[k]);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) out[k * 8 + e] = (float)h[e];  // exact
-    }
-}
-template <int N>
-__device__ __forceinline__ void pack(const float (&in)[N], Packet<float, N>& r) {
-#pragma unroll
-    for (int k = 0; k < N; ++k) r.q[k / 4][k % 4] = in[k];
-}
-// float -> half, round to nearest even (v_cvt_f16_f32 under the default rounding mode).
-// Returns true when a produced half is +-inf or NaN.
-template <int N>
-__device__ __forceinline__ bool pack(const float (&in)[N], Packet<_Float16, N>& r) {
-    bool bad = false;
-#pragma unroll
-    for (int k = 0; k < N / 8; ++k) {
-        f16x8 h;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            h[e] = (_Float16)in[k * 8 + e];
-            const uint16_t bits = __builtin_bit_cast(uint16_t, h[e]);
-            bad |= ((bits & 0x7c00u) == 0x7c00u);
-        }
-        r.q[k] = __builtin_bit_cast(f32x4, h);
-    }
+    for (int k = 0; k < E / 2; ++k) bad |= nonfinite_halves(w[k]);
     return bad;
 }
 
 // The update for one element, all in fp32 registers.
 //   unscaled state: fused_adam_cuda_kernel.cu:115-130     scaled (fp16) state: :94-114
 // out_m/out_v are what gets STORED (already multiplied by optim_scale when kScaled).
-template <bool kScaled>
+template <bool kScaled, int EPS_MODE, bool FAST_SCALES>
 __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, float in_m, float in_v, float in_g,
                                             float& out_p, float& out_m, float& out_v) {
-    const float scaled_grad = (s.flags & kGradScalePow2) ? in_g * s.inv_grad_scale : in_g / s.grad_scale;
+    const float scaled_grad = FAST_SCALES ? in_g * s.inv_grad_scale : in_g / s.grad_scale;
     float momentum, velocity;
     if (kScaled) {
-        const bool pow2 = (s.flags & kOptimScalePow2) != 0;
-        const float m_un = pow2 ? in_m * s.inv_optim_scale : in_m / s.optim_scale;
-        const float v_un = pow2 ? in_v * s.inv_optim_scale : in_v / s.optim_scale;
+        const float m_un = FAST_SCALES ? in_m * s.inv_optim_scale : in_m / s.optim_scale;
+        const float v_un = FAST_SCALES ? in_v * s.inv_optim_scale : in_v / s.optim_scale;
         momentum = s.b1 * m_un + s.one_minus_b1 * scaled_grad;
         velocity = s.b2 * v_un + (s.one_minus_b2 * scaled_grad) * scaled_grad;
         out_m = momentum * s.optim_scale;
@@ -203,169 +173,136 @@ __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, fl
         out_m = momentum;
         out_v = velocity;
     }
-    const float denom = (s.eps_mode == 0) ? sqrtf(velocity + s.eps) : sqrtf(velocity) + s.eps;
+    const float denom = (EPS_MODE == 0) ? sqrtf(velocity + s.eps) : sqrtf(velocity) + s.eps;
     const float update = momentum / denom + s.decay * in_p;
     out_p = in_p - s.step_size * update;
 }
 
-template <typename T>
-__device__ __forceinline__ float load_scalar(gptr<const T> ptr) { return (float)*ptr; }
-__device__ __forceinline__ void store_scalar(gptr<float> ptr, float x) { *ptr = x; }
-__device__ __forceinline__ bool store_scalar(gptr<_Float16> ptr, float x, bool check) {
-    const _Float16 h = (_Float16)x;
-    *ptr = h;
-    return check && ((__builtin_bit_cast(uint16_t, h) & 0x7c00u) == 0x7c00u);
-}
-
-// One element through the element-wise path (tails and misaligned tensors).
-template <int MODE>
-__device__ __forceinline__ bool step_element(const StepScalars& s, gptr<typename ModeTraits<MODE>::P> p,
-                                             gptr<typename ModeTraits<MODE>::S> m, gptr<typename ModeTraits<MODE>::S> v,
-                                             gptr<const typename ModeTraits<MODE>::G> g, gptr<_Float16> p_copy) {
+// A full, aligned tile: GROUPS x (one vector per stream per lane), everything loaded before the
+// first use.  Group k of the tile covers BLOCK*E consecutive elements, lane i the E elements at
+// k*BLOCK*E + i*E, so each instruction of a wave touches one contiguous span.
+template <int MODE, int BLOCK, int GROUPS, int EPS_MODE, bool FAST_SCALES>
+__device__ __forceinline__ uint32_t tile_vector(const ChunkDesc& d, uint32_t off, const StepScalars& s) {
     using T = ModeTraits<MODE>;
-    float np, nm, nv;
-    adam_update<T::kScaled>(s, load_scalar<typename T::P>(p), load_scalar<typename T::S>(m),
-                            load_scalar<typename T::S>(v), load_scalar<typename T::G>(g), np, nm, nv);
-    bool bad = false;
-    if constexpr (sizeof(typename T::S) == 2) {
-        bad |= store_scalar(m, nm, true);
-        bad |= store_scalar(v, nv, true);
-    } else {
-        store_scalar(m, nm);
-        store_scalar(v, nv);
+    using P = typename T::P; using G = typename T::G; using S = typename T::S;
+    constexpr int E = T::kElems;
+    const uint32_t first = off + threadIdx.x * E;
+    gptr<P> p = (gptr<P>)d.p + first;
+    gptr<S> m = (gptr<S>)d.m + first;
+    gptr<S> v = (gptr<S>)d.v + first;
+    gptr<const G> g = (gptr<const G>)d.g + first;
+
+    typename VecOf<P, E>::type rp[GROUPS];
+    typename VecOf<S, E>::type rm[GROUPS], rv[GROUPS];
+    typename VecOf<G, E>::type rg[GROUPS];
+#pragma unroll
+    for (int k = 0; k < GROUPS; ++k) {
+        rp[k] = load_vec<P, E>(p + k * BLOCK * E);
+        rm[k] = load_vec<S, E>(m + k * BLOCK * E);
+        rv[k] = load_vec<S, E>(v + k * BLOCK * E);
+        rg[k] = load_vec<G, E>(g + k * BLOCK * E);
     }
-    if constexpr (sizeof(typename T::P) == 2) {
-        store_scalar(p, np, false);
-    } else {
-        store_scalar(p, np);
-        if constexpr (T::kCopy) store_scalar(p_copy, np, false);  // half(stored fp32 p): kernel.cu:129
+    uint32_t bad = 0;
+#pragma unroll
+    for (int k = 0; k < GROUPS; ++k) {
+        typename VecOf<P, E>::type op;
+        typename VecOf<S, E>::type om, ov;
+        typename VecOf<_Float16, E>::type oc;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float np, nm, nv;
+            adam_update<T::kScaled, EPS_MODE, FAST_SCALES>(s, (float)rp[k][e], (float)rm[k][e], (float)rv[k][e],
+                                                           (float)rg[k][e], np, nm, nv);
+            op[e] = (P)np;  // round to nearest even when P is half
+            om[e] = (S)nm;
+            ov[e] = (S)nv;
+            if constexpr (T::kCopy) oc[e] = (_Float16)np;  // half(stored fp32 p): kernel.cu:129
+        }
+        if constexpr (T::kScaled) bad |= nonfinite_in<E>(om) | nonfinite_in<E>(ov);
+        store_vec<S, E>(m + k * BLOCK * E, om);
+        store_vec<S, E>(v + k * BLOCK * E, ov);
+        store_vec<P, E>(p + k * BLOCK * E, op);
+        if constexpr (T::kCopy) store_vec<_Float16, E>((gptr<_Float16>)d.p_copy + first + k * BLOCK * E, oc);
     }
     return bad;
 }
 
-// kVec consecutive elements of every stream through registers.
-template <int MODE, bool NT>
-struct VectorStep {
+// Ragged or misaligned tile: one element per lane per pass, same arithmetic.
+template <int MODE, int BLOCK, int EPS_MODE, bool FAST_SCALES>
+__device__ __forceinline__ uint32_t tile_elementwise(const ChunkDesc& d, uint32_t off, uint32_t count, const StepScalars& s) {
     using T = ModeTraits<MODE>;
-    static constexpr int kVec = T::kVec;
-    Packet<typename T::P, kVec> rp;
-    Packet<typename T::S, kVec> rm, rv;
-    Packet<typename T::G, kVec> rg;
-
-    __device__ __forceinline__ void load(gptr<const typename T::P> p, gptr<const typename T::S> m,
-                                         gptr<const typename T::S> v, gptr<const typename T::G> g) {
-        rp = load_packet<typename T::P, kVec, NT>(p);
-        rm = load_packet<typename T::S, kVec, NT>(m);
-        rv = load_packet<typename T::S, kVec, NT>(v);
-        rg = load_packet<typename T::G, kVec, NT>(g);
+    using P = typename T::P; using G = typename T::G; using S = typename T::S;
+    gptr<P> p = (gptr<P>)d.p + off;
+    gptr<S> m = (gptr<S>)d.m + off;
+    gptr<S> v = (gptr<S>)d.v + off;
+    gptr<const G> g = (gptr<const G>)d.g + off;
+    gptr<_Float16> pc = T::kCopy ? (gptr<_Float16>)d.p_copy + off : nullptr;
+    uint32_t bad = 0;
+    for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
+        float np, nm, nv;
+        adam_update<T::kScaled, EPS_MODE, FAST_SCALES>(s, (float)p[e], (float)m[e], (float)v[e], (float)g[e], np, nm, nv);
+        const S sm = (S)nm, sv = (S)nv;
+        m[e] = sm;
+        v[e] = sv;
+        if constexpr (T::kScaled)
+            bad |= nonfinite_halves((uint32_t)__builtin_bit_cast(uint16_t, sm) | ((uint32_t)__builtin_bit_cast(uint16_t, sv) << 16));
+        p[e] = (P)np;
+        if constexpr (T::kCopy) pc[e] = (_Float16)np;
     }
-    __device__ __forceinline__ bool compute_store(const StepScalars& s, gptr<typename T::P> p, gptr<typename T::S> m,
-                                                  gptr<typename T::S> v, gptr<_Float16> p_copy) {
-        float fp[kVec], fm[kVec], fv[kVec], fg[kVec];
-        unpack(rp, fp);
-        unpack(rm, fm);
-        unpack(rv, fv);
-        unpack(rg, fg);
-#pragma unroll
-        for (int k = 0; k < kVec; ++k) adam_update<T::kScaled>(s, fp[k], fm[k], fv[k], fg[k], fp[k], fm[k], fv[k]);
-        bool bad = false;
-        Packet<typename T::S, kVec> om, ov;
-        if constexpr (sizeof(typename T::S) == 2) {
-            bad |= pack(fm, om);
-            bad |= pack(fv, ov);
-        } else {
-            pack(fm, om);
-            pack(fv, ov);
-        }
-        store_packet<typename T::S, kVec, NT>(m, om);
-        store_packet<typename T::S, kVec, NT>(v, ov);
-        Packet<typename T::P, kVec> op;
-        pack(fp, op);
-        store_packet<typename T::P, kVec, NT>(p, op);
-        if constexpr (T::kCopy) {
-            Packet<_Float16, kVec> oc;
-            pack(fp, oc);
-            store_packet<_Float16, kVec, NT>(p_copy, oc);
-        }
-        return bad;
-    }
-};
-
-template <int MODE, int UNROLL, bool NT>
-__global__ __launch_bounds__(kBlock) void fsadam_kernel(const TensorRow* __restrict__ table,
-                                                        const uint32_t* __restrict__ chunk_prefix,
-                                                        uint32_t n_tensors, uint32_t n_chunks, uint32_t chunk_elems,
-                                                        StepScalars s, float* __restrict__ found_inf) {
-    using T = ModeTraits<MODE>;
-    constexpr int kVec = T::kVec;
-    extern __shared__ uint32_t lds_prefix[];  // n_tensors + 1 entries, relative to this launch's first chunk
-
-    const uint32_t first = chunk_prefix[0];
-    for (uint32_t i = threadIdx.x; i <= n_tensors; i += kBlock) lds_prefix[i] = chunk_prefix[i] - first;
-    __syncthreads();
-
-    bool bad = false;
-    for (uint32_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        // last tensor t with lds_prefix[t] <= c  (tensors without elements have an empty range and are never hit)
-        uint32_t lo = 0, hi = n_tensors;  // invariant: lds_prefix[lo] <= c < lds_prefix[hi]
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (lds_prefix[mid] <= c) lo = mid; else hi = mid;
-        }
-        const uint32_t t = __builtin_amdgcn_readfirstlane(lo);
-        const uint32_t local_chunk = __builtin_amdgcn_readfirstlane(c - lds_prefix[lo]);
-        const TensorRow row = table[t];
-        const int64_t base = (int64_t)local_chunk * chunk_elems;
-        const int64_t left = row.numel - base;
-        const int n = (int)(left < (int64_t)chunk_elems ? left : (int64_t)chunk_elems);
-
-        gptr<typename T::P> p = (gptr<typename T::P>)row.p + base;
-        gptr<typename T::S> m = (gptr<typename T::S>)row.m + base;
-        gptr<typename T::S> v = (gptr<typename T::S>)row.v + base;
-        gptr<const typename T::G> g = (gptr<const typename T::G>)row.g + base;
-        gptr<_Float16> pc = T::kCopy ? (gptr<_Float16>)row.p_copy + base : nullptr;
-
-        if (row.vector_ok) {
-            const int nvec = n / kVec;
-            int i = threadIdx.x;
-            for (; i + (UNROLL - 1) * kBlock < nvec; i += UNROLL * kBlock) {
-                VectorStep<MODE, NT> st[UNROLL];
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    const int64_t e = (int64_t)(i + u * kBlock) * kVec;
-                    st[u].load(p + e, m + e, v + e, g + e);
-                }
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    const int64_t e = (int64_t)(i + u * kBlock) * kVec;
-                    bad |= st[u].compute_store(s, p + e, m + e, v + e, T::kCopy ? pc + e : nullptr);
-                }
-            }
-            for (; i < nvec; i += kBlock) {
-                VectorStep<MODE, NT> st;
-                const int64_t e = (int64_t)i * kVec;
-                st.load(p + e, m + e, v + e, g + e);
-                bad |= st.compute_store(s, p + e, m + e, v + e, T::kCopy ? pc + e : nullptr);
-            }
-            const int e = nvec * kVec + (int)threadIdx.x;  // fewer than kVec ragged elements at the end of a tensor
-            if (e < n) bad |= step_element<MODE>(s, p + e, m + e, v + e, g + e, T::kCopy ? pc + e : nullptr);
-        } else {
-#pragma unroll 4
-            for (int e = threadIdx.x; e < n; e += kBlock)
-                bad |= step_element<MODE>(s, p + e, m + e, v + e, g + e, T::kCopy ? pc + e : nullptr);
-        }
-    }
-    // Same-value store from every lane that saw a non-finite stored half (kernel.cu:103-105).
-    if (T::kScaled && bad) *(gptr<float>)found_inf = 1.0f;
+    return bad;
 }
 
-__global__ __launch_bounds__(kBlock) void fsadam_copy_kernel(f32x4* __restrict__ dst_, const f32x4* __restrict__ src_,
-                                                             int64_t n_quads) {
+template <int MODE, int BLOCK, int GROUPS, int EPS_MODE, bool FAST_SCALES>
+__device__ __forceinline__ uint32_t tile_any(const ChunkDesc& d, uint32_t off, const StepScalars& s) {
+    constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
+    const uint32_t left = d.n - off;
+    if (d.vector_ok && left >= kTile) return tile_vector<MODE, BLOCK, GROUPS, EPS_MODE, FAST_SCALES>(d, off, s);
+    return tile_elementwise<MODE, BLOCK, EPS_MODE, FAST_SCALES>(d, off, left < kTile ? left : kTile, s);
+}
+
+// One workgroup = one tile.  `log2k`: tiles per descriptor of this launch (0 for the small-tensor
+// launch).  `n_blocks`: tiles really launched for (the grid may be padded for the XCD remap).
+template <int MODE, int BLOCK, int GROUPS>
+__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_blocks,
+                                                      uint32_t xcd_stride, StepScalars s, float* __restrict__ found_inf) {
+    constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
+
+    uint32_t block = blockIdx.x;
+    if (xcd_stride) {
+        // Consecutive workgroups go to consecutive XCDs (eight L2s).  Give XCD x the x-th contiguous
+        // eighth of the tiles instead of every eighth tile.
+        block = (block & 7u) * xcd_stride + (block >> 3);
+        if (block >= n_blocks) return;
+    }
+    const uint32_t chunk = block >> log2k;
+    const uint32_t off = (block & ((1u << log2k) - 1u)) * kTile;
+    // The whole 64-byte descriptor in ONE scalar load (uniform address, constant address space), before
+    // anything is tested: reading the count first and the pointers afterwards would put two memory
+    // latencies in front of the first data load.
+    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
+    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
+        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
+    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    if (off >= d.n) return;  // tile past the end of its tensor (large launch only)
+
+    uint32_t bad;
+    if (s.eps_mode == 0) {
+        bad = s.fast_scales ? tile_any<MODE, BLOCK, GROUPS, 0, true>(d, off, s) : tile_any<MODE, BLOCK, GROUPS, 0, false>(d, off, s);
+    } else {
+        bad = s.fast_scales ? tile_any<MODE, BLOCK, GROUPS, 1, true>(d, off, s) : tile_any<MODE, BLOCK, GROUPS, 1, false>(d, off, s);
+    }
+    // Same-value store from every lane that stored a non-finite fp16 m or v (kernel.cu:103-105).
+    if (ModeTraits<MODE>::kScaled && bad != 0) *(gptr<float>)found_inf = 1.0f;
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fsadam_copy_kernel(f32x4* __restrict__ dst_, const f32x4* __restrict__ src_, int64_t n_quads) {
     gptr<f32x4> dst = (gptr<f32x4>)dst_;
     gptr<const f32x4> src = (gptr<const f32x4>)src_;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_quads; i += stride)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < n_quads) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 // --------------------------------------------------------------------------------------------
@@ -388,20 +325,34 @@ int fail_hip(hipError_t e, const char* what) {
     } while (0)
 
 struct Options {
-    int64_t chunk_elems = 16384;
-    int64_t wg_per_cu = 8;
-    int64_t nontemporal = 1;
-    int64_t unroll = 2;
+    int64_t block = 64;         // threads per workgroup: 64, 128 or 256
+    int64_t groups = 1;         // vectors per lane per stream: 1 or 2
+    int64_t lds_throttle = -1;  // bytes of untouched LDS per workgroup (0 = no cap, -1 = per-mode default)
+    int64_t xcd_remap = 0;      // 1: contiguous eighth of the tiles per XCD
 };
+
+// Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
+// about 40-48 KiB of loads in flight per compute unit, i.e. 10 waves of the 4 KiB-per-wave modes and
+// 12 of the 3-3.5 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
+int64_t default_lds_throttle(int mode) {
+    switch (mode) {
+        case FSADAM_FULL_PRECISION: return 16384;
+        case FSADAM_MIXED_PRECISION: return 16384;
+        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 13312;
+        default: return 13312;
+    }
+}
 Options g_opt;
 std::mutex g_mutex;        // guards g_opt
 std::mutex g_cache_mutex;  // guards the fsadam_step table cache
 
 bool valid_mode(int mode) { return mode >= FSADAM_FULL_PRECISION && mode <= FSADAM_PURE_FP16; }
 
-int elem_size_p(int mode) { return (mode == FSADAM_FULL_PRECISION || mode == FSADAM_MIXED_PRECISION) ? 4 : 2; }
+int size_p(int mode) { return (mode == FSADAM_FULL_PRECISION || mode == FSADAM_MIXED_PRECISION) ? 4 : 2; }
+int size_s(int mode) { return mode == FSADAM_PURE_FP16 ? 2 : 4; }
+int size_g(int mode) { return mode == FSADAM_FULL_PRECISION ? 4 : 2; }
 
-bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+bool aligned_to(const void* ptr, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(ptr) & (bytes - 1)) == 0; }
 
 bool is_pow2_with_exact_reciprocal(float x, float* inv) {
     if (!(x > 0.0f) || !std::isfinite(x)) return false;
@@ -425,86 +376,154 @@ int validate_rows(const FsAdamTensor* tensors, int64_t n, int mode) {
         if (!r.p || !r.m || !r.v || !r.g) return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": NULL p/m/v/g pointer");
         if (mode == FSADAM_MIXED_PRECISION && !r.p_copy)
             return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": MIXED_PRECISION needs p_copy");
-        // element alignment: anything less cannot be a tensor of that dtype
-        const uintptr_t pa = elem_size_p(mode) - 1, sa = (mode == FSADAM_PURE_FP16 ? 2 : 4) - 1,
-                        ga = (mode == FSADAM_FULL_PRECISION ? 4 : 2) - 1;
-        if ((reinterpret_cast<uintptr_t>(r.p) & pa) || (reinterpret_cast<uintptr_t>(r.m) & sa) ||
-            (reinterpret_cast<uintptr_t>(r.v) & sa) || (reinterpret_cast<uintptr_t>(r.g) & ga) ||
-            (mode == FSADAM_MIXED_PRECISION && (reinterpret_cast<uintptr_t>(r.p_copy) & 1)))
+        // anything less than element alignment cannot be a tensor of that dtype
+        if (!aligned_to(r.p, size_p(mode)) || !aligned_to(r.m, size_s(mode)) || !aligned_to(r.v, size_s(mode)) ||
+            !aligned_to(r.g, size_g(mode)) || (mode == FSADAM_MIXED_PRECISION && !aligned_to(r.p_copy, 2)))
             return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": pointer not aligned to its element size");
     }
     return FSADAM_OK;
 }
 
+// The vector path moves kElems elements per lane per instruction: each stream must be aligned to that.
 bool row_vector_ok(const FsAdamTensor& r, int mode) {
-    return aligned16(r.p) && aligned16(r.m) && aligned16(r.v) && aligned16(r.g) &&
-           (mode != FSADAM_MIXED_PRECISION || aligned16(r.p_copy));
+    const uintptr_t e = mode_elems(mode);
+    return aligned_to(r.p, e * size_p(mode)) && aligned_to(r.m, e * size_s(mode)) && aligned_to(r.v, e * size_s(mode)) &&
+           aligned_to(r.g, e * size_g(mode)) && (mode != FSADAM_MIXED_PRECISION || aligned_to(r.p_copy, e * 2));
 }
 
-int64_t chunks_of(int64_t numel, int64_t chunk_elems) { return (numel + chunk_elems - 1) / chunk_elems; }
+int64_t floor_pow2(int64_t x) {
+    int64_t p = 1;
+    while (p * 2 <= x) p *= 2;
+    return p;
+}
+int log2_exact(int64_t x) {
+    int k = 0;
+    while ((int64_t(1) << k) < x) ++k;
+    return k;
+}
+
+// How a tensor list is cut into descriptors for given options.
+struct Layout {
+    int64_t tile_elems = 0;
+    int64_t large_chunk_elems = 0;
+    int64_t n_large = 0, n_small = 0, n_empty = 0;
+    int64_t n_large_descs = 0, n_small_descs = 0;
+    int64_t total_elems = 0;
+    int64_t n_vector = 0, n_scalar = 0;
+};
+
+int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Options& opt) {
+    Layout L;
+    L.tile_elems = opt.block * mode_elems(mode) * opt.groups;
+    int64_t min_large = 0;
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t numel = tensors[t].numel;
+        L.total_elems += numel;
+        if (numel == 0) { L.n_empty += 1; continue; }
+        (row_vector_ok(tensors[t], mode) ? L.n_vector : L.n_scalar) += 1;
+        if (numel >= kLargeThreshold) {
+            L.n_large += 1;
+            if (min_large == 0 || numel < min_large) min_large = numel;
+        } else {
+            L.n_small += 1;
+        }
+    }
+    // every large tensor spans at least two chunks, so the empty tiles after its end stay a small share
+    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t numel = tensors[t].numel;
+        if (numel == 0) continue;
+        if (numel >= kLargeThreshold) L.n_large_descs += ceil_div(numel, L.large_chunk_elems);
+        else L.n_small_descs += ceil_div(numel, L.tile_elems);
+    }
+    return L;
+}
 
 }  // namespace
 
 struct FsAdamPlan {
     int mode = 0;
     int device = -1;
-    int cu_count = 0;
     Options opt;
+    Layout layout;
     std::vector<FsAdamTensor> rows;  // what the device table was built from
-    int64_t total_elems = 0, total_chunks = 0, n_vector = 0, n_scalar = 0, uploads = 0;
-    // one device allocation: TensorRow[cap_tensors] then uint32_t[cap_tensors + 1]
-    int64_t cap_tensors = 0;
-    void* d_buf = nullptr;
-    void* h_buf = nullptr;  // pinned staging of the same layout
+    int64_t uploads = 0;
+    int64_t cap_descs = 0;  // capacity of d_table / h_table, in descriptors
+    ChunkDesc* d_table = nullptr;
+    ChunkDesc* h_table = nullptr;  // pinned staging
     hipEvent_t last_use = nullptr;
     bool used = false;
     uint64_t lru = 0;  // fsadam_step cache bookkeeping
-
-    TensorRow* d_rows() const { return static_cast<TensorRow*>(d_buf); }
-    uint32_t* d_prefix() const { return reinterpret_cast<uint32_t*>(static_cast<char*>(d_buf) + cap_tensors * sizeof(TensorRow)); }
-    TensorRow* h_rows() const { return static_cast<TensorRow*>(h_buf); }
-    uint32_t* h_prefix() const { return reinterpret_cast<uint32_t*>(static_cast<char*>(h_buf) + cap_tensors * sizeof(TensorRow)); }
-    size_t buf_bytes() const { return cap_tensors * sizeof(TensorRow) + (cap_tensors + 1) * sizeof(uint32_t); }
 };
 
 namespace {
 
-int plan_release_buffers(FsAdamPlan* plan) {
+void plan_release_buffers(FsAdamPlan* plan) {
     if (plan->used && plan->last_use) (void)hipEventSynchronize(plan->last_use);
-    if (plan->d_buf) (void)hipFree(plan->d_buf);
-    if (plan->h_buf) (void)hipHostFree(plan->h_buf);
-    plan->d_buf = plan->h_buf = nullptr;
-    plan->cap_tensors = 0;
+    if (plan->d_table) (void)hipFree(plan->d_table);
+    if (plan->h_table) (void)hipHostFree(plan->h_table);
+    plan->d_table = plan->h_table = nullptr;
+    plan->cap_descs = 0;
+}
+
+char* advance(const void* base, int64_t elems, int elem_size) {
+    return const_cast<char*>(static_cast<const char*>(base)) + elems * elem_size;
+}
+
+void fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t chunk_elems, bool vec) {
+    const int64_t chunks = ceil_div(r.numel, chunk_elems);
+    for (int64_t c = 0; c < chunks; ++c) {
+        const int64_t first = c * chunk_elems;
+        ChunkDesc& d = out[c];
+        d.p = advance(r.p, first, size_p(mode));
+        d.m = advance(r.m, first, size_s(mode));
+        d.v = advance(r.v, first, size_s(mode));
+        d.g = advance(r.g, first, size_g(mode));
+        d.p_copy = (mode == FSADAM_MIXED_PRECISION) ? advance(r.p_copy, first, 2) : nullptr;
+        d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - first);
+        d.vector_ok = vec ? 1u : 0u;
+        d.pad = 0;
+    }
+}
+
+template <int MODE, int BLOCK, int GROUPS>
+int launch_tiles(const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s,
+                 float* found_inf, hipStream_t stream) {
+    if (n_descs == 0) return FSADAM_OK;
+    const int64_t n_blocks = n_descs << log2k;
+    if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
+    uint32_t grid = (uint32_t)n_blocks, xcd_stride = 0;
+    if (opt.xcd_remap) {
+        xcd_stride = (uint32_t)ceil_div(n_blocks, 8);
+        grid = xcd_stride * 8;
+    }
+    hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table,
+                       (uint32_t)log2k, (uint32_t)n_blocks, xcd_stride, s, found_inf);
+    FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
 
 template <int MODE>
-int launch_mode(const FsAdamPlan* plan, const StepScalars& s, float* found_inf, hipStream_t stream) {
-    const int64_t n = (int64_t)plan->rows.size();
-    const uint32_t* hp = plan->h_prefix();
-    for (int64_t t0 = 0; t0 < n; t0 += kWindow) {
-        const int64_t nt = std::min<int64_t>(kWindow, n - t0);
-        const uint32_t n_chunks = hp[t0 + nt] - hp[t0];
-        if (n_chunks == 0) continue;
-        const int64_t want = (int64_t)plan->cu_count * plan->opt.wg_per_cu;
-        const uint32_t grid = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(n_chunks, want));
-        const size_t lds = (size_t)(nt + 1) * sizeof(uint32_t);
-        const TensorRow* rows = plan->d_rows() + t0;
-        const uint32_t* prefix = plan->d_prefix() + t0;
-        const uint32_t chunk_elems = (uint32_t)plan->opt.chunk_elems;
-#define FS_LAUNCH(U, NT)                                                                                    \
-    hipLaunchKernelGGL((fsadam_kernel<MODE, U, NT>), dim3(grid), dim3(kBlock), lds, stream, rows, prefix, \
-                       (uint32_t)nt, n_chunks, chunk_elems, s, found_inf)
-        const bool nt_hint = plan->opt.nontemporal != 0;
-        switch (plan->opt.unroll) {
-            case 1: if (nt_hint) FS_LAUNCH(1, true); else FS_LAUNCH(1, false); break;
-            case 4: if (nt_hint) FS_LAUNCH(4, true); else FS_LAUNCH(4, false); break;
-            default: if (nt_hint) FS_LAUNCH(2, true); else FS_LAUNCH(2, false); break;
-        }
-#undef FS_LAUNCH
-        FS_HIP(hipGetLastError());
+int launch_shape(const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s, float* found_inf,
+                 hipStream_t stream) {
+#define FS_CASE(B, G) \
+    if (opt.block == B && opt.groups == G) return launch_tiles<MODE, B, G>(table, n_descs, log2k, opt, s, found_inf, stream)
+    FS_CASE(64, 1); FS_CASE(64, 2); FS_CASE(128, 1); FS_CASE(128, 2); FS_CASE(256, 1); FS_CASE(256, 2);
+#undef FS_CASE
+    return fail(FSADAM_EINVAL, "unsupported block/groups combination");
+}
+
+int launch_mode(int mode, const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s,
+                float* found_inf, hipStream_t stream) {
+    switch (mode) {
+        case FSADAM_FULL_PRECISION: return launch_shape<FSADAM_FULL_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
+        case FSADAM_MIXED_PRECISION: return launch_shape<FSADAM_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
+        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION:
+            return launch_shape<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
+        default: return launch_shape<FSADAM_PURE_FP16>(table, n_descs, log2k, opt, s, found_inf, stream);
     }
-    return FSADAM_OK;
 }
 
 int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, hipStream_t stream) {
@@ -513,55 +532,55 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     if (plan->device != dev) {
-        if (plan->d_buf) plan_release_buffers(plan);
+        plan_release_buffers(plan);
         plan->device = dev;
-        FS_HIP(hipDeviceGetAttribute(&plan->cu_count, hipDeviceAttributeMultiprocessorCount, dev));
-        if (plan->cu_count < 1) return fail(FSADAM_ENODEVICE, "device reports no compute units");
         if (!plan->last_use) FS_HIP(hipEventCreateWithFlags(&plan->last_use, hipEventDisableTiming));
     }
     {
         std::lock_guard<std::mutex> lock(g_mutex);
         plan->opt = g_opt;
     }
-    const int64_t chunk_elems = plan->opt.chunk_elems;
-    uint64_t chunks = 0;
-    for (int64_t t = 0; t < n; ++t) chunks += (uint64_t)chunks_of(tensors[t].numel, chunk_elems);
-    if (chunks > 0xffffffffull) return fail(FSADAM_EINVAL, "tensor list needs more than 2^32 chunks; raise chunk_elems");
+    if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
+    const Layout L = compute_layout(tensors, n, plan->mode, plan->opt);
+    const int64_t n_descs = L.n_large_descs + L.n_small_descs;
+    if (L.n_large_descs * (L.large_chunk_elems / L.tile_elems) > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0)
+        return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
     // the previous table may still be read by a kernel in flight
     if (plan->used) FS_HIP(hipEventSynchronize(plan->last_use));
-    if (n > plan->cap_tensors) {
+    if (n_descs > plan->cap_descs) {
         plan_release_buffers(plan);
-        plan->cap_tensors = std::max<int64_t>(n, 16);
-        if (hipMalloc(&plan->d_buf, plan->buf_bytes()) != hipSuccess) {
-            plan->d_buf = nullptr; plan->cap_tensors = 0;
-            return fail(FSADAM_ENOMEM, "hipMalloc of the tensor table failed");
+        const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
+        if (hipMalloc(reinterpret_cast<void**>(&plan->d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
+            plan->d_table = nullptr;
+            return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
         }
-        if (hipHostMalloc(&plan->h_buf, plan->buf_bytes(), hipHostMallocDefault) != hipSuccess) {
-            (void)hipFree(plan->d_buf);
-            plan->d_buf = plan->h_buf = nullptr; plan->cap_tensors = 0;
-            return fail(FSADAM_ENOMEM, "hipHostMalloc of the table staging buffer failed");
+        if (hipHostMalloc(reinterpret_cast<void**>(&plan->h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
+            (void)hipFree(plan->d_table);
+            plan->d_table = plan->h_table = nullptr;
+            return fail(FSADAM_ENOMEM, "hipHostMalloc of the descriptor staging buffer failed");
         }
+        plan->cap_descs = cap;
     }
-    TensorRow* hr = plan->h_rows();
-    uint32_t* hp = plan->h_prefix();
-    plan->total_elems = 0; plan->n_vector = 0; plan->n_scalar = 0;
-    uint32_t run = 0;
+    // large tensors first (one launch), then small ones (second launch)
+    ChunkDesc* large = plan->h_table;
+    ChunkDesc* small = plan->h_table + L.n_large_descs;
     for (int64_t t = 0; t < n; ++t) {
         const FsAdamTensor& r = tensors[t];
-        const bool vec = r.numel > 0 && row_vector_ok(r, plan->mode);
-        hr[t] = TensorRow{r.p, r.m, r.v, r.g, r.p_copy, r.numel, vec ? 1u : 0u, 0u};
-        hp[t] = run;
-        run += (uint32_t)chunks_of(r.numel, chunk_elems);
-        plan->total_elems += r.numel;
-        if (r.numel > 0) (vec ? plan->n_vector : plan->n_scalar) += 1;
+        if (r.numel == 0) continue;
+        const bool vec = row_vector_ok(r, plan->mode);
+        if (r.numel >= kLargeThreshold) {
+            fill_descs(large, r, plan->mode, L.large_chunk_elems, vec);
+            large += ceil_div(r.numel, L.large_chunk_elems);
+        } else {
+            fill_descs(small, r, plan->mode, L.tile_elems, vec);
+            small += ceil_div(r.numel, L.tile_elems);
+        }
     }
-    hp[n] = run;
-    plan->total_chunks = run;
+    plan->layout = L;
     plan->rows.assign(tensors, tensors + n);
-    // rows and prefix are not adjacent when n < cap_tensors: two copies
-    FS_HIP(hipMemcpyAsync(plan->d_rows(), hr, (size_t)n * sizeof(TensorRow), hipMemcpyHostToDevice, stream));
-    FS_HIP(hipMemcpyAsync(plan->d_prefix(), hp, (size_t)(n + 1) * sizeof(uint32_t), hipMemcpyHostToDevice, stream));
+    if (n_descs > 0)
+        FS_HIP(hipMemcpyAsync(plan->d_table, plan->h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
     FS_HIP(hipEventRecord(plan->last_use, stream));
     plan->used = true;
     plan->uploads += 1;
@@ -570,13 +589,14 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
 
 int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, float grad_scale, float optim_scale,
               float decay, int step, int eps_mode, int bias_correction, float* found_inf, hipStream_t stream) {
-    if (plan->rows.empty() || !plan->d_buf) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
+    if (plan->rows.empty()) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
     if (eps_mode != FSADAM_EPS_INSIDE_SQRT && eps_mode != FSADAM_EPS_OUTSIDE_SQRT)
         return fail(FSADAM_EINVAL, "eps_mode must be 0 (inside sqrt) or 1 (outside)");
     if (plan->mode == FSADAM_PURE_FP16 && !found_inf) return fail(FSADAM_EINVAL, "PURE_FP16 needs a found_inf device pointer");
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
-    if (dev != plan->device) return fail(FSADAM_EINVAL, "plan belongs to device " + std::to_string(plan->device) + ", current device is " + std::to_string(dev));
+    if (dev != plan->device)
+        return fail(FSADAM_EINVAL, "plan belongs to device " + std::to_string(plan->device) + ", current device is " + std::to_string(dev));
 
     StepScalars s;
     s.b1 = beta1; s.b2 = beta2;
@@ -587,17 +607,15 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     s.grad_scale = grad_scale; s.optim_scale = optim_scale;
     s.inv_grad_scale = 0.f; s.inv_optim_scale = 0.f;
     s.eps_mode = eps_mode;
-    s.flags = 0;
-    if (is_pow2_with_exact_reciprocal(grad_scale, &s.inv_grad_scale)) s.flags |= kGradScalePow2;
-    if (is_pow2_with_exact_reciprocal(optim_scale, &s.inv_optim_scale)) s.flags |= kOptimScalePow2;
+    const bool gs_ok = is_pow2_with_exact_reciprocal(grad_scale, &s.inv_grad_scale);
+    const bool os_ok = is_pow2_with_exact_reciprocal(optim_scale, &s.inv_optim_scale);
+    s.fast_scales = (gs_ok && (plan->mode != FSADAM_PURE_FP16 || os_ok)) ? 1 : 0;
 
-    int rc;
-    switch (plan->mode) {
-        case FSADAM_FULL_PRECISION: rc = launch_mode<FSADAM_FULL_PRECISION>(plan, s, found_inf, stream); break;
-        case FSADAM_MIXED_PRECISION: rc = launch_mode<FSADAM_MIXED_PRECISION>(plan, s, found_inf, stream); break;
-        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: rc = launch_mode<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION>(plan, s, found_inf, stream); break;
-        default: rc = launch_mode<FSADAM_PURE_FP16>(plan, s, found_inf, stream); break;
-    }
+    const Layout& L = plan->layout;
+    const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
+    int rc = launch_mode(plan->mode, plan->d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
+    if (rc) return rc;
+    rc = launch_mode(plan->mode, plan->d_table + L.n_large_descs, L.n_small_descs, 0, plan->opt, s, found_inf, stream);
     if (rc) return rc;
     FS_HIP(hipEventRecord(plan->last_use, stream));
     return FSADAM_OK;
@@ -615,6 +633,10 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
         if (a.p != b.p || a.m != b.m || a.v != b.v || a.g != b.g || a.p_copy != b.p_copy || a.numel != b.numel) return false;
     }
     return true;
+}
+
+bool same_options(const Options& a, const Options& b) {
+    return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap;
 }
 
 }  // namespace
@@ -641,18 +663,18 @@ int fsadam_set_option(const char* name, int64_t value) {
     if (!name) return fail(FSADAM_EINVAL, "option name is NULL");
     std::lock_guard<std::mutex> lock(g_mutex);
     const std::string k(name);
-    if (k == "chunk_elems") {
-        if (value < kChunkQuantum || value % kChunkQuantum || value > (1 << 30)) return fail(FSADAM_EINVAL, "chunk_elems must be a multiple of 2048 in [2048, 2^30]");
-        g_opt.chunk_elems = value;
-    } else if (k == "wg_per_cu") {
-        if (value < 1 || value > (1 << 24)) return fail(FSADAM_EINVAL, "wg_per_cu must be in [1, 2^24]");
-        g_opt.wg_per_cu = value;
-    } else if (k == "nontemporal") {
-        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "nontemporal must be 0 or 1");
-        g_opt.nontemporal = value;
-    } else if (k == "unroll") {
-        if (value != 1 && value != 2 && value != 4) return fail(FSADAM_EINVAL, "unroll must be 1, 2 or 4");
-        g_opt.unroll = value;
+    if (k == "block") {
+        if (value != 64 && value != 128 && value != 256) return fail(FSADAM_EINVAL, "block must be 64, 128 or 256");
+        g_opt.block = value;
+    } else if (k == "groups") {
+        if (value != 1 && value != 2) return fail(FSADAM_EINVAL, "groups must be 1 or 2");
+        g_opt.groups = value;
+    } else if (k == "lds_throttle") {
+        if (value < -1 || value > 65536) return fail(FSADAM_EINVAL, "lds_throttle must be -1 (per-mode default) or in [0, 65536] bytes");
+        g_opt.lds_throttle = value;
+    } else if (k == "xcd_remap") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "xcd_remap must be 0 or 1");
+        g_opt.xcd_remap = value;
     } else {
         return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
     }
@@ -663,27 +685,38 @@ int fsadam_get_option(const char* name, int64_t* value) {
     if (!name || !value) return fail(FSADAM_EINVAL, "NULL argument");
     std::lock_guard<std::mutex> lock(g_mutex);
     const std::string k(name);
-    if (k == "chunk_elems") *value = g_opt.chunk_elems;
-    else if (k == "wg_per_cu") *value = g_opt.wg_per_cu;
-    else if (k == "nontemporal") *value = g_opt.nontemporal;
-    else if (k == "unroll") *value = g_opt.unroll;
+    if (k == "block") *value = g_opt.block;
+    else if (k == "groups") *value = g_opt.groups;
+    else if (k == "lds_throttle") *value = g_opt.lds_throttle;
+    else if (k == "xcd_remap") *value = g_opt.xcd_remap;
     else return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
     return FSADAM_OK;
 }
 
-int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, int64_t chunk_elems,
-                  uint64_t* chunk_prefix, uint8_t* vector_ok) {
+int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out, uint8_t* tensor_class,
+                  uint8_t* vector_ok) {
     int rc = validate_rows(tensors, n_tensors, precision_mode);
     if (rc) return rc;
-    if (chunk_elems < kChunkQuantum || chunk_elems % kChunkQuantum) return fail(FSADAM_EINVAL, "chunk_elems must be a positive multiple of 2048");
-    if (!chunk_prefix || !vector_ok) return fail(FSADAM_EINVAL, "NULL output");
-    uint64_t run = 0;
-    for (int64_t t = 0; t < n_tensors; ++t) {
-        chunk_prefix[t] = run;
-        run += (uint64_t)chunks_of(tensors[t].numel, chunk_elems);
-        vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode)) ? 1 : 0;
+    if (!out) return fail(FSADAM_EINVAL, "out is NULL");
+    Options opt;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        opt = g_opt;
     }
-    chunk_prefix[n_tensors] = run;
+    const Layout L = compute_layout(tensors, n_tensors, precision_mode, opt);
+    out->tile_elems = L.tile_elems;
+    out->large_chunk_elems = L.large_chunk_elems;
+    out->n_large_tensors = L.n_large;
+    out->n_small_tensors = L.n_small;
+    out->n_empty_tensors = L.n_empty;
+    out->n_large_descriptors = L.n_large_descs;
+    out->n_small_descriptors = L.n_small_descs;
+    out->grid_large = L.n_large_descs * (L.large_chunk_elems / L.tile_elems);
+    out->grid_small = L.n_small_descs;
+    for (int64_t t = 0; t < n_tensors; ++t) {
+        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (tensors[t].numel >= kLargeThreshold ? 2 : 1);
+        if (vector_ok) vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode)) ? 1 : 0;
+    }
     return FSADAM_OK;
 }
 
@@ -713,28 +746,20 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
 int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
     if (!plan || !out) return fail(FSADAM_EINVAL, "NULL argument");
     std::memset(out, 0, sizeof(*out));
+    const Layout& L = plan->layout;
     out->mode = plan->mode;
     out->device = plan->device;
     out->n_tensors = (int64_t)plan->rows.size();
-    out->total_elems = plan->total_elems;
-    out->total_chunks = plan->total_chunks;
-    out->chunk_elems = plan->opt.chunk_elems;
-    out->n_vector_tensors = plan->n_vector;
-    out->n_scalar_tensors = plan->n_scalar;
-    out->n_launches = 0;
-    out->grid = 0;
-    if (plan->h_buf) {
-        const int64_t n = (int64_t)plan->rows.size();
-        const uint32_t* hp = plan->h_prefix();
-        for (int64_t t0 = 0; t0 < n; t0 += kWindow) {
-            const int64_t nt = std::min<int64_t>(kWindow, n - t0);
-            const uint32_t n_chunks = hp[t0 + nt] - hp[t0];
-            if (!n_chunks) continue;
-            if (out->n_launches == 0) out->grid = std::max<int64_t>(1, std::min<int64_t>(n_chunks, (int64_t)plan->cu_count * plan->opt.wg_per_cu));
-            out->n_launches += 1;
-        }
-    }
-    out->block = kBlock;
+    out->total_elems = L.total_elems;
+    out->tile_elems = L.tile_elems;
+    out->large_chunk_elems = L.large_chunk_elems;
+    out->n_descriptors = L.n_large_descs + L.n_small_descs;
+    out->n_vector_tensors = L.n_vector;
+    out->n_scalar_tensors = L.n_scalar;
+    out->n_launches = (L.n_large_descs > 0) + (L.n_small_descs > 0);
+    out->grid = L.tile_elems ? L.n_large_descs * (L.large_chunk_elems / L.tile_elems) + L.n_small_descs : 0;
+    out->block = plan->opt.block;
+    out->lds_throttle = plan->opt.lds_throttle;
     out->uploads = plan->uploads;
     return FSADAM_OK;
 }
@@ -755,11 +780,17 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    Options now;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        now = g_opt;
+    }
+    if (now.lds_throttle < 0) now.lds_throttle = default_lds_throttle(precision_mode);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     FsAdamPlan* hit = nullptr;
     FsAdamPlan* victim = nullptr;
     for (FsAdamPlan* c : g_cache) {
-        if (c->device == dev && c->mode == precision_mode && same_rows(c, tensors, n_tensors)) { hit = c; break; }
+        if (c->device == dev && c->mode == precision_mode && same_options(c->opt, now) && same_rows(c, tensors, n_tensors)) { hit = c; break; }
         if (c->mode == precision_mode && (c->device == dev || c->device < 0) && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -794,15 +825,13 @@ int fsadam_clear_cache(void) {
 }
 
 int fsadam_calib_copy(void* dst, const void* src, int64_t nbytes, void* hip_stream) {
-    if (!dst || !src || nbytes < 0 || (nbytes & 15) || !aligned16(dst) || !aligned16(src))
+    if (!dst || !src || nbytes < 0 || (nbytes & 15) || !aligned_to(dst, 16) || !aligned_to(src, 16))
         return fail(FSADAM_EINVAL, "calib copy needs 16-byte aligned pointers and a multiple of 16 bytes");
     if (nbytes == 0) return FSADAM_OK;
-    int dev = -1, cus = 0;
-    FS_HIP(hipGetDevice(&dev));
-    FS_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int64_t quads = nbytes / 16;
-    const int64_t grid = std::max<int64_t>(1, std::min<int64_t>((quads + kBlock - 1) / kBlock, (int64_t)cus * 8));
-    hipLaunchKernelGGL(fsadam_copy_kernel, dim3((uint32_t)grid), dim3(kBlock), 0, static_cast<hipStream_t>(hip_stream),
+    const int64_t grid = ceil_div(quads, 64);
+    if (grid > 0x7fffffff) return fail(FSADAM_EINVAL, "calib copy larger than 2^31 wavefronts");
+    hipLaunchKernelGGL(fsadam_copy_kernel<64>, dim3((uint32_t)grid), dim3(64), 20480, static_cast<hipStream_t>(hip_stream),
                        static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), quads);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;

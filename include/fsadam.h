@@ -63,15 +63,30 @@ typedef struct FsAdamPlanInfo {
     int32_t device;
     int64_t n_tensors;
     int64_t total_elems;
-    int64_t total_chunks;     /* work items of chunk_elems elements (last one of a tensor may be short) */
-    int64_t chunk_elems;
-    int64_t n_vector_tensors; /* tensors whose every stream is 16-byte aligned: 128-bit path          */
-    int64_t n_scalar_tensors; /* tensors taking the element-wise path because of a misaligned stream  */
-    int64_t n_launches;       /* kernel launches one step needs (1 unless n_tensors > table window)   */
-    int64_t grid;             /* workgroups of the first launch                                       */
-    int64_t block;            /* threads per workgroup                                                */
-    int64_t uploads;          /* how many times the table has been (re)sent to the device             */
+    int64_t tile_elems;        /* elements one workgroup handles                                        */
+    int64_t large_chunk_elems; /* elements per shared descriptor of a large tensor                      */
+    int64_t n_descriptors;     /* 64-byte rows of the device table                                      */
+    int64_t n_vector_tensors;  /* tensors whose every stream is aligned for the 64/128-bit vector path  */
+    int64_t n_scalar_tensors;  /* tensors taking the element-wise path because of a misaligned stream   */
+    int64_t n_launches;        /* kernel launches per step: 0, 1 or 2                                   */
+    int64_t grid;              /* workgroups per step, all launches                                     */
+    int64_t block;             /* threads per workgroup                                                 */
+    int64_t lds_throttle;      /* bytes of LDS ballast per workgroup                                    */
+    int64_t uploads;           /* how many times the table has been (re)sent to the device              */
 } FsAdamPlanInfo;
+
+/* How fsadam_plan_set_tensors would cut a tensor list into descriptors (see fsadam_layout). */
+typedef struct FsAdamLayout {
+    int64_t tile_elems;
+    int64_t large_chunk_elems;
+    int64_t n_large_tensors;     /* numel >= 131072: descriptors shared by large_chunk_elems/tile_elems tiles */
+    int64_t n_small_tensors;     /* one descriptor per tile                                                   */
+    int64_t n_empty_tensors;     /* numel == 0: skipped                                                       */
+    int64_t n_large_descriptors;
+    int64_t n_small_descriptors;
+    int64_t grid_large;          /* workgroups of the large-tensor launch (some past a tensor's end: they exit) */
+    int64_t grid_small;          /* workgroups of the small-tensor launch                                      */
+} FsAdamLayout;
 
 /* ---- library ---- */
 
@@ -87,9 +102,12 @@ const char* fsadam_last_error(void);
 float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_correction);
 
 /* Tuning knobs, by name; returns FSADAM_EINVAL for an unknown name or a value out of range.
- *   "chunk_elems"   elements per work item (multiple of 2048, default 16384)
- *   "wg_per_cu"     resident workgroups requested per compute unit (default 8)
- *   "nontemporal"   0/1: non-temporal hint on streaming loads and stores (default 1)
+ *   "block"         threads per workgroup: 64, 128 or 256 (default 64)
+ *   "groups"        vectors per lane per stream: 1 or 2 (default 1)
+ *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
+ *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
+ *                   per-mode default (13-16 KiB, default)
+ *   "xcd_remap"     0/1: hand each XCD a contiguous eighth of the tiles (default 0)
  * Affects plans whose tensors are set after the call. */
 int fsadam_set_option(const char* name, int64_t value);
 int fsadam_get_option(const char* name, int64_t* value);
@@ -124,11 +142,11 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
 int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out);
 int fsadam_plan_destroy(FsAdamPlan* plan);
 
-/* Host-only planning (no device needed): fills chunk_prefix[n_tensors+1] (exclusive prefix sum of
- * per-tensor chunk counts) and vector_ok[n_tensors] (1 = every stream 16-byte aligned) the way
- * fsadam_plan_set_tensors lays the table out for `chunk_elems`. */
-int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, int64_t chunk_elems,
-                  uint64_t* chunk_prefix, uint8_t* vector_ok);
+/* Host-only planning (no device needed): how the list would be laid out under the current options.
+ * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large.  vector_ok[n_tensors] (may be
+ * NULL): 1 = every stream aligned for the vector path. */
+int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
+                  uint8_t* tensor_class, uint8_t* vector_ok);
 
 /* Drops the tables cached by fsadam_step (synchronises the devices that own them). */
 int fsadam_clear_cache(void);

@@ -113,6 +113,14 @@ uint16_t oracle_float_to_half(float f) { /* round to nearest, ties to even */
     return (uint16_t)(sign | (base + kept));
 }
 
+void oracle_float_to_half_array(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = oracle_float_to_half(in[i]);
+}
+
+void oracle_half_to_float_array(const uint16_t* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = oracle_half_to_float(in[i]);
+}
+
 /* ---- step size, fused_adam_cuda_kernel.cu:153-162 ----
  * std::pow(float, int) promotes to double; "1 - pow" is a double subtraction that is then narrowed
  * to float; sqrt, multiply and divide are float operations evaluated left to right. */

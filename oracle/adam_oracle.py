@@ -71,6 +71,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_half_to_float.restype = f32
         L.oracle_half_to_float.argtypes = [ctypes.c_uint16]
         L.fsadam_oracle_threads.restype = i32
+        L.oracle_float_to_half_array.restype = None
+        L.oracle_float_to_half_array.argtypes = [vp, vp, i64]
+        L.oracle_half_to_float_array.restype = None
+        L.oracle_half_to_float_array.argtypes = [vp, vp, i64]
         _lib = L
     return _lib
 
@@ -89,6 +93,21 @@ def float_to_half_c(x: float) -> int:
 
 def half_to_float_c(h: int) -> np.float32:
     return np.float32(lib().oracle_half_to_float(h))
+
+
+def float_to_half_array_c(x: np.ndarray) -> np.ndarray:
+    """float32 array -> uint16 array of half bit patterns, through the C oracle's software conversion."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().oracle_float_to_half_array(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
+def half_to_float_array_c(h: np.ndarray) -> np.ndarray:
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().oracle_half_to_float_array(h.ctypes.data, out.ctypes.data, h.size)
+    return out
 
 
 def _check(arr: np.ndarray, dtype, name: str) -> None:

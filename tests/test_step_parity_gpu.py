@@ -113,8 +113,10 @@ def test_c1_full_precision_flat_2pow20(oracle, cuda_device):
 @pytest.mark.parametrize("bias_correction", [0, 1])
 def test_modes_edge_sizes(oracle, cuda_device, mode, eps_mode, bias_correction):
     """Every dtype combination x eps placement x bias correction over sizes around every boundary
-    the kernel has: vector width (4/8), workgroup pass, chunk (16384) and the reference's 65536."""
-    sizes = [1, 2, 3, 4, 5, 7, 8, 9, 15, 17, 255, 2047, 2048, 2049, 4095, 4097, 16383, 16384, 16385, 32769, 65535, 65536, 65537, 100003]
+    the kernel has: vector width (4/8), tile (256..4096), the reference's 65536 chunk, the
+    small/large tensor threshold (131072) and a large tensor that ends just into a shared chunk."""
+    sizes = [1, 2, 3, 4, 5, 7, 8, 9, 15, 17, 255, 256, 257, 511, 513, 1023, 1025, 2047, 2048, 2049, 4095, 4097, 16383, 16384, 16385,
+             32769, 65535, 65536, 65537, 100003, 131071, 131072, 131073, 196611, 262144 + 5]
     hyper = dict(DEFAULT, eps_mode=eps_mode, bias_correction=bias_correction, decay=0.01)
     gs = 1.0 if mode == FULL else 1024.0
     run_case(oracle, cuda_device, mode, sizes, 3, 4000 + mode, hyper, grad_scale=gs, optim_scale=65536.0 if mode == PURE16 else 1.0)
@@ -131,9 +133,9 @@ def test_non_power_of_two_scales(oracle, cuda_device, mode):
 @pytest.mark.parametrize("which", ["p", "g", "m", "all"])
 def test_misaligned_views(oracle, cuda_device, mode, which):
     """Views that start 1 element (p: 3) into an allocation, like OSS bucket views: a stream that is
-    not 16-byte aligned sends the tensor down the element-wise path; results must not change."""
+    not aligned for the vector path sends the tensor down the element-wise path; results must not change."""
     mis = {"p": {"p": 3}, "g": {"g": 1}, "m": {"m": 1}, "all": {"p": 1, "g": 1, "m": 1, "v": 1, "p16": 1}}[which]
-    run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
+    run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000, 140001], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
              grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
@@ -141,8 +143,8 @@ def test_zero_sized_tensors_in_list(oracle, cuda_device):
     run_case(oracle, cuda_device, FULL, [0, 5, 0, 0, 20000, 0], 2, 4300, DEFAULT)
 
 
-def test_more_tensors_than_one_table_window(oracle, cuda_device):
-    """9000 small tensors: more than the 8192 rows one launch stages in LDS, so two launches."""
+def test_nine_thousand_tiny_tensors(oracle, cuda_device):
+    """9000 tensors of 1..37 elements: one descriptor and one ragged tile each, all in the small-tensor launch."""
     sizes = [(i % 37) + 1 for i in range(9000)]
     run_case(oracle, cuda_device, MEMEFF, sizes, 2, 4400, dict(DEFAULT, decay=0.01), grad_scale=64.0)
 
@@ -214,6 +216,31 @@ def test_pure_fp16_flag_set_exactly_when_state_overflows(oracle, cuda_device):
     kw["step"] = 3
     dev.step(g, **kw)
     assert dev.found_inf.item() == 1.0  # sticky: the caller clears it (adam.py:256)
+
+
+@pytest.mark.parametrize("misaligned", [False, True])
+def test_pure_fp16_flag_for_every_position_in_a_vector(oracle, cuda_device, misaligned):
+    """One overflowing element at a time, at every position of a 128-bit packet (8 halves), in the
+    ragged tail, in the first and the last chunk: the flag must go up each time, and stay down for
+    the clean control.  Guards the in-kernel check against being applied to only part of a packet."""
+    n = 3 * 1024 + 8 * 5 + 3  # a few whole tiles, a few whole vectors and a 3-element tail
+    positions = list(range(0, 8)) + list(range(1024 - 8, 1024 + 8)) + list(range(n - 11, n)) + [None]
+    kw = dict(DEFAULT, step=1, optim_scale=65536.0)
+    for pos in positions:
+        host = C.Tensors(PURE16, [n], 4700)
+        dev = GpuList(host, cuda_device, {"m": 1} if misaligned else None)
+        g = host.grads(1)
+        if pos is not None:
+            g[0][pos] = np.float16(6e4)
+        dev.step(g, **kw)
+        flag = np.zeros(1, np.float32)
+        oracle_step(oracle, host, g, flag, **kw)
+        compare(host, dev, f"overflow at {pos}")
+        want = 0.0 if pos is None else 1.0
+        assert flag[0] == want
+        assert dev.found_inf.item() == want, f"overflow injected at element {pos} (misaligned={misaligned})"
+        nonfinite = (~torch.isfinite(dev.m[0])).any().item() or (~torch.isfinite(dev.v[0])).any().item()
+        assert nonfinite == (pos is not None)
 
 
 def test_flat_vs_split_is_bitwise_identical(cuda_device):
