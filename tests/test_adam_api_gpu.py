@@ -1,0 +1,345 @@
+"""GPU tests of ``fairscale_amd.optim.Adam``: the behaviours ``tests/optim/test_adam.py`` of the
+reference pins (precision inference, state dtypes, state_dict round trips, optimizer-state-scale
+transitions, error types), plus whole trajectories against the oracle's host state machine."""
+from __future__ import annotations
+
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import _cases as C
+from _cases import FULL, MEMEFF, MIXED, PURE16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    torch.manual_seed(1)
+    yield
+
+
+@pytest.fixture(scope="module")
+def api(cuda_device):
+    from fairscale_amd.optim import Adam, GradScaler, Precision
+
+    return Adam, GradScaler, Precision
+
+
+def tiny_problem(dtype, device):
+    """loss = sum((W x + b)^2) for a 2x1 weight, like the reference's tests."""
+    weight = torch.randn(2, 1).to(device=device, dtype=dtype).requires_grad_()
+    bias = torch.randn(2).to(device=device, dtype=dtype).requires_grad_()
+    x = torch.randn(1).to(device=device, dtype=dtype)
+    return weight, bias, x
+
+
+def closure_for(opt, weight, bias, x):
+    def fn():
+        opt.zero_grad()
+        loss = (weight.mv(x) + bias).pow(2).sum()
+        loss.backward()
+        return loss
+
+    return fn
+
+
+def loss_goes_down(opt, weight, bias, x, steps=5):
+    repr(opt)
+    fn = closure_for(opt, weight, bias, x)
+    first = fn().item()
+    for _ in range(steps):
+        opt.step(fn)
+    return fn().item() < first
+
+
+def state_dtypes(opt, params):
+    return {opt.state[p][k].dtype for p in params for k in ("exp_avg", "exp_avg_sq")}
+
+
+# ---- precision modes (test_adam.py:111-195)
+
+def test_full_precision_is_inferred_from_fp32_parameters(api, cuda_device):
+    Adam, _, Precision = api
+    w, b, x = tiny_problem(torch.float32, cuda_device)
+    opt = Adam([w, b], lr=1e-3)
+    assert opt.precision is Precision.FULL_PRECISION and opt.optim_type == torch.float32
+    assert loss_goes_down(opt, w, b, x)
+    assert not opt.fp32_param_groups and not opt.mixed_precision
+    assert state_dtypes(opt, [w, b]) == {torch.float32}
+    assert w.dtype == torch.float32
+
+
+def test_mixed_precision_is_inferred_from_fp16_parameters(api, cuda_device):
+    Adam, _, Precision = api
+    w, b, x = tiny_problem(torch.float16, cuda_device)
+    opt = Adam([w, b], lr=1e-3)
+    assert opt.precision is Precision.MIXED_PRECISION and opt.mixed_precision
+    assert loss_goes_down(opt, w, b, x)
+    assert len(opt.fp32_param_groups) == len(opt.param_groups) == 1
+    for master, half in zip(opt.fp32_param_groups[0]["params"], opt.param_groups[0]["params"]):
+        assert master.dtype == torch.float32 and half.dtype == torch.float16
+        assert (master.detach() - half.detach().float()).abs().max().item() < 1e-3
+        assert torch.equal(master.detach().half(), half.detach())  # the copy-out is half(master), exactly
+    assert state_dtypes(opt, [w, b]) == {torch.float32}
+
+
+def test_memory_efficient_keeps_fp16_params_and_fp32_state(api, cuda_device):
+    Adam, _, Precision = api
+    w, b, x = tiny_problem(torch.float16, cuda_device)
+    opt = Adam([w, b], lr=1e-3, precision=Precision.MEMORY_EFFICIENT_MIXED_PRECISION)
+    assert loss_goes_down(opt, w, b, x)
+    assert w.dtype == torch.float16 and not opt.fp32_param_groups
+    assert state_dtypes(opt, [w, b]) == {torch.float32}
+
+
+def test_pure_fp16_keeps_everything_in_fp16(api, cuda_device):
+    Adam, _, Precision = api
+    w, b, x = tiny_problem(torch.float16, cuda_device)
+    opt = Adam([w, b], lr=1e-3, precision=Precision.PURE_FP16)
+    assert opt.optim_type == torch.float16 and opt._optim_scale == 2.0 ** 16
+    assert loss_goes_down(opt, w, b, x)
+    assert w.dtype == torch.float16 and not opt.fp32_param_groups
+    assert state_dtypes(opt, [w, b]) == {torch.float16}
+
+
+def test_properties_and_defaults(api, cuda_device):
+    Adam, _, _ = api
+    w, b, _ = tiny_problem(torch.float32, cuda_device)
+    opt = Adam([w, b])
+    assert opt.supports_memory_efficient_fp16 is True and opt._step_supports_amp_scaling is False
+    assert opt.defaults == {"lr": 1e-3, "bias_correction": True, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0.0, "max_grad_norm": 0.0}
+    assert opt.eps_mode == 1 and Adam([w, b], eps_inside_sqrt=True).eps_mode == 0
+    assert opt._optim_scale == 1.0 and opt._optim_scale_update_freq == 2000 and opt._steps_since_optim_scale_change == 0
+    assert opt._overflow_buf.dtype == torch.int32 and opt._overflow_buf.is_cuda
+
+
+def test_works_with_grad_scaler(api, cuda_device):  # test_adam.py:242-259
+    Adam, GradScaler, Precision = api
+    w, b, x = tiny_problem(torch.float16, cuda_device)
+    opt = Adam([w, b], lr=1e-3, precision=Precision.PURE_FP16)
+    scaler = GradScaler()
+    first = None
+    for i in range(5):
+        opt.zero_grad()
+        loss = (w.mv(x) + b).pow(2).sum()
+        if i == 0:
+            first = loss.item()
+        scaler.scale(loss).backward()
+        scaler.step(opt)
+        scaler.update()
+    assert loss.item() < first
+
+
+# ---- state_dict (test_adam.py:64-103, 262-305)
+
+@pytest.mark.parametrize("precision_name", ["FULL_PRECISION", "PURE_FP16", "MIXED_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION"])
+def test_state_dict_round_trip_keeps_lock_step(api, cuda_device, precision_name):
+    """Save after 5 steps, load into a fresh optimizer on cloned weights: m and v are equal and five
+    more steps side by side stay bitwise equal.  The two mixed modes are expected failures in the
+    reference (its load casts fp32 state through fp16); here the state is restored exactly."""
+    Adam, _, Precision = api
+    precision = getattr(Precision, precision_name)
+    dtype = torch.float32 if precision is Precision.FULL_PRECISION else torch.float16
+    w, b, x = tiny_problem(dtype, cuda_device)
+    opt = Adam([w, b], lr=1e-3, precision=precision)
+    fn = closure_for(opt, w, b, x)
+    for _ in range(5):
+        opt.step(fn)
+    w2 = w.data.clone().requires_grad_()
+    b2 = b.data.clone().requires_grad_()
+    opt2 = Adam([w2, b2], lr=1e-3, precision=precision)
+    sd = copy.deepcopy(opt.state_dict())
+    assert sd["optim_scale"] == opt._optim_scale
+    opt2.load_state_dict(sd)
+    for p, q in ((w, w2), (b, b2)):
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert opt2.state[q][key].dtype == opt.optim_type
+            assert torch.equal(opt.state[p][key], opt2.state[q][key])
+        assert opt2.state[q]["step"] == opt.state[p]["step"] == 5
+    if opt.fp32_param_groups:  # masters are rebuilt from fp16, not saved (test_adam.py:90-95)
+        opt2.fp32_param_groups = copy.deepcopy(opt.fp32_param_groups)
+    fn2 = closure_for(opt2, w2, b2, x)
+    for _ in range(5):
+        opt.step(fn)
+        opt2.step(fn2)
+        assert torch.equal(w, w2) and torch.equal(b, b2)
+
+
+# ---- optimizer-state scale (test_adam.py:308-337)
+
+def test_optim_scale_grows_after_a_clean_interval(api, cuda_device):
+    Adam, _, Precision = api
+    w, b, x = tiny_problem(torch.float16, cuda_device)
+    opt = Adam([w, b], lr=1e-3, precision=Precision.PURE_FP16)
+    opt._optim_scale_update_freq = 1
+    opt._optim_scale = 2 ** 15
+    closure_for(opt, w, b, x)()
+    opt.step()
+    assert opt._optim_scale == 2 ** 16
+    closure_for(opt, w, b, x)()
+    opt.step()
+    assert opt._optim_scale == 2 ** 16  # capped
+
+
+def test_exploding_state_raises_when_scale_drops_below_one(api, cuda_device):
+    Adam, _, Precision = api
+    w = torch.tensor([[float("inf")]]).half().to(cuda_device).requires_grad_()
+    x = torch.tensor([1.0]).half().to(cuda_device).requires_grad_()
+    opt = Adam([w], lr=1e-3, precision=Precision.PURE_FP16)
+    opt._optim_scale = 1.0
+    opt.zero_grad()
+    w.mv(x).pow(2).sum().backward()
+    with pytest.raises(RuntimeError, match="Optimizer state scale < 1"):
+        opt.step()
+
+
+def test_build_fp32_params_can_be_called_again(api, cuda_device):
+    Adam, _, _ = api
+    w = torch.randn(10, 5).to(cuda_device).half().requires_grad_()
+    b = torch.randn(10).to(cuda_device).half().requires_grad_()
+    opt = Adam([w, b], lr=1e-3)
+    opt._build_fp32_params([w, b])
+    assert len(opt.fp32_param_groups) == 1
+    for master, half in zip(opt.fp32_param_groups[0]["params"], [w, b]):
+        assert master.dtype == torch.float32 and master.grad is not None
+        assert torch.equal(master.detach(), half.detach().float())
+
+
+# ---- constructor errors (test_adam.py:355-406)
+
+def test_constructor_errors(api, cuda_device):
+    Adam, _, Precision = api
+    w = torch.randn(10, 5, device=cuda_device, requires_grad=True)
+    b = torch.randn(10, device=cuda_device, requires_grad=True)
+    with pytest.raises(ValueError):
+        Adam([w, b], lr=1e-2, betas=(1.0, 0.0))
+    with pytest.raises(ValueError):
+        Adam([w, b], lr=1e-2, weight_decay=-1)
+    with pytest.raises(RuntimeError, match="AMSGrad"):
+        Adam([w, b], lr=1e-2, amsgrad=True)
+    for precision in (Precision.MIXED_PRECISION, Precision.MEMORY_EFFICIENT_MIXED_PRECISION, Precision.PURE_FP16):
+        with pytest.raises(AssertionError):
+            Adam([w, b], lr=1e-2, precision=precision)
+
+
+def test_step_without_any_gradient_raises_index_error(api, cuda_device):
+    Adam, _, _ = api
+    w, b, _ = tiny_problem(torch.float32, cuda_device)
+    with pytest.raises(IndexError):  # adam.py:256 indexes an empty dict's first key
+        Adam([w, b]).step()
+
+
+def test_sparse_gradients_are_refused(api, cuda_device):
+    Adam, _, _ = api
+    w = torch.randn(4, 3, device=cuda_device, requires_grad=True)
+    w.grad = torch.zeros(4, 3, device=cuda_device).to_sparse()
+    with pytest.raises(RuntimeError, match="sparse"):
+        Adam([w]).step()
+
+
+# ---- whole trajectories against the oracle's host state machine
+
+MODE_OF = {"FULL_PRECISION": FULL, "MIXED_PRECISION": MIXED, "MEMORY_EFFICIENT_MIXED_PRECISION": MEMEFF, "PURE_FP16": PURE16}
+
+
+@pytest.mark.parametrize("precision_name", list(MODE_OF))
+def test_trajectory_matches_oracle_state_machine(oracle, api, cuda_device, precision_name):
+    """8 steps over a ragged list with weight decay, a parameter that never gets a gradient, a
+    parameter whose gradient is missing on some steps and (PURE_FP16) an overflow on step 4: params,
+    m, v, step counters and the optimizer-state scale must follow the oracle exactly."""
+    Adam, _, Precision = api
+    mode = MODE_OF[precision_name]
+    pd, gd, _ = C.MODE_DTYPES[mode]
+    host_dtype = np.float16 if mode != FULL else np.float32
+    sizes = [3, 1000, 4097, 70000, 150001]
+    rng = np.random.default_rng(80 + mode)
+    host = [(rng.standard_normal(n).astype(np.float32) * 0.02).astype(host_dtype) for n in sizes]
+    params = [torch.from_numpy(h.copy()).to(cuda_device).requires_grad_() for h in host]
+    opt = Adam(params, lr=2e-3, betas=(0.8, 0.99), eps=1e-6, weight_decay=0.02, precision=getattr(Precision, precision_name))
+    ref = oracle.OracleAdam([h.copy() for h in host], mode, lr=2e-3, betas=(0.8, 0.99), eps=1e-6, weight_decay=0.02)
+    opt._optim_scale_update_freq = ref.optim_scale_update_freq = 3
+    for step in range(1, 9):
+        grads = []
+        for j, n in enumerate(sizes):
+            if j == 0 or (j == 2 and step % 3 == 0):
+                grads.append(None)  # never / sometimes without a gradient (adam.py:212)
+                continue
+            g = (rng.standard_normal(n).astype(np.float32) * 1e-3).astype(gd)
+            if mode == PURE16 and step == 4 and j == 3:
+                g[12345] = np.float16(6e4)
+            grads.append(g)
+        for p, g in zip(params, grads):
+            p.grad = None if g is None else torch.from_numpy(g).to(cuda_device)
+        opt.step()
+        ref.step(grads)
+        assert opt._optim_scale == ref.optim_scale, f"step {step}"
+        assert opt._steps_since_optim_scale_change == ref.steps_since_optim_scale_change
+        for j, p in enumerate(params):
+            assert np.array_equal(p.detach().cpu().numpy().view(np.uint8), ref.params[j].view(np.uint8)), f"step {step} param {j}"
+            if ref.state[j].get("step") is not None:
+                st = opt.state[p]
+                assert st["step"] == ref.state[j]["step"]
+                for key in ("exp_avg", "exp_avg_sq"):
+                    assert np.array_equal(st[key].cpu().numpy().view(np.uint8), ref.state[j][key].view(np.uint8)), f"step {step} {key}[{j}]"
+        if mode == MIXED:
+            for j, master in enumerate(opt.fp32_param_groups[0]["params"]):
+                assert np.array_equal(master.detach().cpu().numpy(), ref.fp32_params[j])
+    if mode == PURE16:
+        assert opt._optim_scale < 2.0 ** 16 or ref.optim_scale == 2.0 ** 16  # it backed off at step 4 (and may have regrown)
+    assert len(opt.state[params[0]]) == 0  # a parameter that never had a gradient keeps an empty state
+
+
+def test_scale_keyword_divides_the_gradients(oracle, api, cuda_device):
+    """step(scale=s) on gradients multiplied by s gives the bits of step() on the plain gradients."""
+    Adam, _, Precision = api
+    rng = np.random.default_rng(90)
+    h = (rng.standard_normal(5000).astype(np.float32) * 0.02).astype(np.float16)
+    g = (rng.standard_normal(5000).astype(np.float32) * 1e-3).astype(np.float16)
+    g = np.where(np.abs(g.astype(np.float32)) < 1e-4, np.float16(1e-3), g)  # keep halves normal at both scales
+    outs = []
+    for s in (1.0, 1024.0):
+        p = torch.from_numpy(h.copy()).to(cuda_device).requires_grad_()
+        opt = Adam([p], precision=Precision.MEMORY_EFFICIENT_MIXED_PRECISION)
+        p.grad = torch.from_numpy((g.astype(np.float32) * s).astype(np.float16)).to(cuda_device)
+        opt.step(scale=s)
+        outs.append((p.detach().clone(), opt.state[p]["exp_avg"].clone(), opt.state[p]["exp_avg_sq"].clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
+def test_table_is_sent_again_only_when_a_pointer_moves(api, cuda_device):
+    Adam, _, _ = api
+    params = [torch.randn(n, device=cuda_device).requires_grad_() for n in (10, 3000, 200000)]
+    opt = Adam(params)
+    grads = [torch.randn_like(p) * 1e-3 for p in params]
+    for p, g in zip(params, grads):
+        p.grad = g
+    for _ in range(3):
+        opt.step()
+    plan = next(iter(opt._plans.values()))
+    info = plan.info()
+    assert info["uploads"] == 1 and info["n_tensors"] == 3 and info["n_launches"] == 2 and info["n_vector_tensors"] == 3
+    params[1].grad = torch.randn_like(params[1]) * 1e-3  # a fresh gradient tensor: its pointer moves
+    opt.step()
+    assert plan.info()["uploads"] == 2
+    opt.step()
+    assert plan.info()["uploads"] == 2
+
+
+def test_native_call_checks_list_shapes_on_device(cuda_device):
+    from fairscale_amd import fused_adam_hip
+
+    mk = lambda *ns: [torch.zeros(n, device=cuda_device) for n in ns]  # noqa: E731
+    flag = torch.zeros(1, device=cuda_device)
+    call = lambda lists: fused_adam_hip.adam(65536, None, lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)  # noqa: E731
+    with pytest.raises(RuntimeError, match="Size mismatch among tensor lists"):
+        call([mk(4, 5), mk(4), mk(4, 5), mk(4, 5)])
+    with pytest.raises(RuntimeError, match="Size mismatch"):
+        call([mk(4, 5), mk(4, 6), mk(4, 5), mk(4, 5)])
+    with pytest.raises(RuntimeError, match="found_inf"):
+        fused_adam_hip.adam(65536, None, [mk(4)] * 4, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, torch.zeros(1), 1, 1, 1, 0.0)
+    call([mk(4, 5), mk(4, 5), mk(4, 5), mk(4, 5)])  # and a well-formed call goes through
+    torch.cuda.synchronize()

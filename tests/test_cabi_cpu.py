@@ -1,0 +1,247 @@
+"""CPU-only checks of the C ABI and the host logic around it: the library loads, exports what
+include/fsadam.h declares, rounds the step size like the oracle, plans tensor lists as documented and
+rejects bad arguments with error codes -- no kernel is launched and no device is touched."""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from fairscale_amd import _cabi, fused_adam_hip
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = open(os.path.join(REPO, "include", "fsadam.h")).read()
+
+
+def declared_functions():
+    code = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"\b(fsadam_[a-z_0-9]+)\s*\(", code)))
+
+
+def header_define(name):
+    m = re.search(r"#define\s+%s\s+\(?(-?\d+)\)?" % name, HEADER)
+    assert m, name
+    return int(m.group(1))
+
+
+def rows(*tensors):
+    """FsAdamTensor array from (p, m, v, g, p_copy, numel) tuples of plain integers."""
+    arr = (_cabi.FsAdamTensor * len(tensors))()
+    for r, t in zip(arr, tensors):
+        r.p, r.m, r.v, r.g, r.p_copy, r.numel = t
+    return arr
+
+
+def last_error():
+    return _cabi.lib().fsadam_last_error().decode()
+
+
+def test_library_exports_every_declared_symbol():
+    L = _cabi.lib()
+    names = declared_functions()
+    assert len(names) >= 14
+    for name in names:
+        assert hasattr(L, name), f"{name} is declared in include/fsadam.h but not exported by libfsadam.so"
+    assert sorted(_cabi.SIGNATURES) == names, "the ctypes binding and the header disagree on the function list"
+
+
+def test_abi_version_and_constants():
+    assert _cabi.lib().fsadam_version() == header_define("FSADAM_ABI_VERSION") == _cabi.ABI_VERSION
+    from oracle import adam_oracle as O
+
+    for name, a, b in [("FSADAM_FULL_PRECISION", _cabi.FULL_PRECISION, O.FULL_PRECISION),
+                       ("FSADAM_MIXED_PRECISION", _cabi.MIXED_PRECISION, O.MIXED_PRECISION),
+                       ("FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION", _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, O.MEMORY_EFFICIENT_MIXED_PRECISION),
+                       ("FSADAM_PURE_FP16", _cabi.PURE_FP16, O.PURE_FP16)]:
+        assert header_define(name) == a == b
+    assert header_define("FSADAM_EPS_INSIDE_SQRT") == 0 and header_define("FSADAM_EPS_OUTSIDE_SQRT") == 1
+    assert ctypes.sizeof(_cabi.FsAdamTensor) == 48  # five pointers and an int64, no padding
+
+
+def test_step_size_is_bit_identical_to_the_oracle(oracle):
+    for lr in (1e-3, 3e-4, 0.1, 1.0):
+        for b1, b2 in ((0.9, 0.999), (0.95, 0.98), (0.0, 0.5), (0.5, 0.9)):
+            for step in (1, 2, 3, 7, 100, 2000, 123456):
+                for bc in (0, 1):
+                    got = np.float32(_cabi.step_size(lr, b1, b2, step, bc))
+                    want = oracle.step_size_c(lr, b1, b2, step, bc)
+                    assert got.view(np.uint32) == np.float32(want).view(np.uint32), (lr, b1, b2, step, bc)
+
+
+def test_options_roundtrip_and_validation():
+    old = {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap")}
+    try:
+        _cabi.set_option("block", 128)
+        _cabi.set_option("groups", 2)
+        _cabi.set_option("lds_throttle", 20480)
+        assert (_cabi.get_option("block"), _cabi.get_option("groups"), _cabi.get_option("lds_throttle")) == (128, 2, 20480)
+        for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", 2), ("no_such_option", 1)):
+            with pytest.raises(_cabi.FsAdamError):
+                _cabi.set_option(name, bad)
+    finally:
+        for k, v in old.items():
+            _cabi.set_option(k, v)
+
+
+def layout(tensors, mode):
+    arr = rows(*tensors)
+    out = _cabi.FsAdamLayout()
+    cls = (ctypes.c_uint8 * len(tensors))()
+    vec = (ctypes.c_uint8 * len(tensors))()
+    _cabi.check(_cabi.lib().fsadam_layout(arr, len(tensors), mode, ctypes.byref(out), cls, vec))
+    return out.as_dict(), list(cls), list(vec)
+
+
+def test_layout_classes_and_descriptor_counts():
+    A = 0x7000_0000_0000  # fake, 2 MiB-aligned device addresses: never dereferenced on the host
+    t = lambda n, off=0: (A + off, A + (1 << 32), A + (2 << 32), A + (3 << 32) + off, 0, n)  # noqa: E731
+    old = {k: _cabi.get_option(k) for k in ("block", "groups")}
+    try:
+        _cabi.set_option("block", 64)
+        _cabi.set_option("groups", 1)
+        lay, cls, vec = layout([t(0), t(1), t(255), t(256), t(257), t(131071), t(131072), t(131073), t(1 << 20)], _cabi.FULL_PRECISION)
+        assert lay["tile_elems"] == 256  # 64 lanes x 4 fp32
+        assert cls == [0, 1, 1, 1, 1, 1, 2, 2, 2]
+        assert lay["n_empty_tensors"] == 1 and lay["n_small_tensors"] == 5 and lay["n_large_tensors"] == 3
+        # smallest large tensor has 131072 elements: chunk = 65536 (two chunks each at least)
+        assert lay["large_chunk_elems"] == 65536
+        assert lay["n_small_descriptors"] == 1 + 1 + 1 + 2 + 512
+        assert lay["n_large_descriptors"] == 2 + 3 + 16
+        assert lay["grid_large"] == lay["n_large_descriptors"] * (65536 // 256)
+        assert lay["grid_small"] == lay["n_small_descriptors"]
+        assert vec == [0, 1, 1, 1, 1, 1, 1, 1, 1]
+        # one 1.63e9-element tensor: chunk capped at 2^24, 98 descriptors
+        lay, cls, _ = layout([t(1_630_000_000)], _cabi.MEMORY_EFFICIENT_MIXED_PRECISION)
+        assert lay["large_chunk_elems"] == 1 << 24 and lay["n_large_descriptors"] == 98 and cls == [2]
+        # PURE_FP16 moves 8 halves per lane
+        lay, _, _ = layout([t(5000)], _cabi.PURE_FP16)
+        assert lay["tile_elems"] == 512 and lay["n_small_descriptors"] == 10
+        _cabi.set_option("block", 256)
+        _cabi.set_option("groups", 2)
+        lay, _, _ = layout([t(5000)], _cabi.FULL_PRECISION)
+        assert lay["tile_elems"] == 2048 and lay["n_small_descriptors"] == 3
+    finally:
+        for k, v in old.items():
+            _cabi.set_option(k, v)
+
+
+def test_layout_alignment_rule_per_mode():
+    A = 0x7000_0000_0000
+    n = 1000
+
+    def vec_ok(mode, p=0, m=0, v=0, g=0, pc=0):
+        _, _, vec = layout([(A + p, A + (1 << 32) + m, A + (2 << 32) + v, A + (3 << 32) + g, A + (4 << 32) + pc, n)], mode)
+        return vec[0]
+
+    # fp32 streams need 16 bytes; fp16 streams need 8 bytes in the 4-element modes and 16 in PURE_FP16
+    assert vec_ok(_cabi.FULL_PRECISION) == 1
+    for k in ("p", "m", "v", "g"):
+        assert vec_ok(_cabi.FULL_PRECISION, **{k: 4}) == 0 and vec_ok(_cabi.FULL_PRECISION, **{k: 16}) == 1
+    assert vec_ok(_cabi.MIXED_PRECISION, g=8) == 1 and vec_ok(_cabi.MIXED_PRECISION, g=2) == 0
+    assert vec_ok(_cabi.MIXED_PRECISION, pc=8) == 1 and vec_ok(_cabi.MIXED_PRECISION, pc=6) == 0 and vec_ok(_cabi.MIXED_PRECISION, p=8) == 0
+    assert vec_ok(_cabi.MEMORY_EFFICIENT_MIXED_PRECISION, p=8, g=8) == 1 and vec_ok(_cabi.MEMORY_EFFICIENT_MIXED_PRECISION, m=8) == 0
+    assert vec_ok(_cabi.PURE_FP16, p=8) == 0 and vec_ok(_cabi.PURE_FP16, p=16, m=16, v=16, g=16) == 1
+
+
+def test_bad_arguments_return_einval_before_touching_a_device():
+    L = _cabi.lib()
+    A = 0x7000_0000_0000
+    good = (A, A + 4096, A + 8192, A + 12288, 0, 16)
+    args = (1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, 0.0, 1, 1, 1, None, None)
+    EINVAL = header_define("FSADAM_EINVAL")
+    cases = [
+        (rows(good), 0, _cabi.FULL_PRECISION, "empty"),               # multi_tensor_apply.cuh:51
+        (rows(good), 1, 7, "unknown precision mode"),
+        (None, 1, _cabi.FULL_PRECISION, "NULL"),
+        (rows((A, A, A, A, 0, -5)), 1, _cabi.FULL_PRECISION, "negative numel"),
+        (rows((0, A, A, A, 0, 16)), 1, _cabi.FULL_PRECISION, "NULL p/m/v/g"),
+        (rows((A, A, A, A + 2, 0, 16)), 1, _cabi.FULL_PRECISION, "not aligned to its element size"),
+        (rows((A, A, A, A + 1, 0, 16)), 1, _cabi.PURE_FP16, "not aligned to its element size"),
+        (rows(good), 1, _cabi.MIXED_PRECISION, "needs p_copy"),
+    ]
+    for arr, n, mode, needle in cases:
+        rc = L.fsadam_step(arr, n, mode, *args)
+        assert rc == EINVAL, needle
+        assert needle in last_error()
+    out = _cabi.FsAdamLayout()
+    assert L.fsadam_layout(rows(good), 1, 9, ctypes.byref(out), None, None) == EINVAL
+    assert L.fsadam_layout(rows(good), 1, 0, None, None, None) == EINVAL
+
+
+def test_plan_lifecycle_without_a_device():
+    L = _cabi.lib()
+    EINVAL = header_define("FSADAM_EINVAL")
+    handle = ctypes.c_void_p()
+    assert L.fsadam_plan_create(5, ctypes.byref(handle)) == EINVAL
+    assert L.fsadam_plan_create(_cabi.PURE_FP16, None) == EINVAL
+    _cabi.check(L.fsadam_plan_create(_cabi.PURE_FP16, ctypes.byref(handle)))
+    info = _cabi.FsAdamPlanInfo()
+    _cabi.check(L.fsadam_plan_info(handle, ctypes.byref(info)))
+    assert info.mode == _cabi.PURE_FP16 and info.n_tensors == 0 and info.uploads == 0 and info.n_launches == 0
+    # stepping a plan that has no tensors is an argument error, not a crash
+    assert L.fsadam_plan_step(handle, 1e-3, 0.9, 0.999, 1e-8, 1.0, 65536.0, 0.0, 1, 1, 1, None, None) == EINVAL
+    assert "no tensors" in last_error()
+    assert L.fsadam_plan_set_tensors(handle, None, 1, None) == EINVAL
+    _cabi.check(L.fsadam_plan_destroy(handle))
+    _cabi.check(L.fsadam_plan_destroy(None))
+    _cabi.check(L.fsadam_clear_cache())
+    assert L.fsadam_calib_copy(None, None, 16, None) == EINVAL
+    assert L.fsadam_calib_copy(ctypes.c_void_p(4096), ctypes.c_void_p(8192), 24, None) == EINVAL
+
+
+# ---- the Python face of the native call (validation of multi_tensor_apply.cuh:49-67, dispatch of kernel.cu:165-263)
+
+def _lists(p_dtype, g_dtype, s_dtype, n=8, copy=False):
+    mk = lambda dt: [torch.zeros(n, dtype=dt), torch.zeros(3, dtype=dt)]  # noqa: E731
+    out = [mk(p_dtype), mk(s_dtype), mk(s_dtype), mk(g_dtype)]
+    if copy:
+        out.append(mk(torch.float16))
+    return out
+
+
+def test_mode_dispatch_follows_the_reference():
+    f32, f16 = torch.float32, torch.float16
+    assert fused_adam_hip.mode_of_lists(_lists(f32, f32, f32)) == _cabi.FULL_PRECISION
+    assert fused_adam_hip.mode_of_lists(_lists(f32, f16, f32, copy=True)) == _cabi.MIXED_PRECISION
+    assert fused_adam_hip.mode_of_lists(_lists(f16, f16, f32)) == _cabi.MEMORY_EFFICIENT_MIXED_PRECISION
+    assert fused_adam_hip.mode_of_lists(_lists(f16, f16, f16)) == _cabi.PURE_FP16
+    for bad in (_lists(f32, f16, f32), _lists(f32, f32, f16), _lists(torch.bfloat16, torch.bfloat16, f32),
+                _lists(f16, f16, torch.float64), _lists(f32, f32, f32, copy=True), _lists(f32, f32, f32)[:3], [[], [], [], []]):
+        with pytest.raises(RuntimeError):
+            fused_adam_hip.mode_of_lists(bad)
+
+
+def test_list_validation_raises_runtime_error_like_torch_check():
+    flag = torch.zeros(1)
+    call = lambda lists: fused_adam_hip.adam(65536, None, lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)  # noqa: E731
+    with pytest.raises(RuntimeError, match="not cuda"):
+        call(_lists(torch.float32, torch.float32, torch.float32))
+    # same order as the reference: contiguity is checked before the device (multi_tensor_apply.cuh:59-64)
+    lists = _lists(torch.float32, torch.float32, torch.float32)
+    lists[0][0] = torch.zeros(16)[::2]
+    with pytest.raises(RuntimeError, match="not contiguous"):
+        call(lists)
+
+
+def test_rows_of_lists_matches_the_struct_layout():
+    lists = _lists(torch.float32, torch.float16, torch.float32, copy=True)
+    arr = fused_adam_hip.rows_of_lists(lists)
+    assert arr.shape == (2, 6) and arr.dtype == np.int64 and arr.flags["C_CONTIGUOUS"]
+    view = ctypes.cast(arr.ctypes.data, ctypes.POINTER(_cabi.FsAdamTensor))
+    for t in range(2):
+        assert view[t].p == lists[0][t].data_ptr() and view[t].m == lists[1][t].data_ptr()
+        assert view[t].v == lists[2][t].data_ptr() and view[t].g == lists[3][t].data_ptr()
+        assert view[t].p_copy == lists[4][t].data_ptr() and view[t].numel == lists[0][t].numel()
+
+
+def test_optimizer_module_imports_and_exposes_the_reference_names():
+    import fairscale_amd.optim as fo
+
+    assert [p.name for p in fo.Precision] == ["FULL_PRECISION", "MIXED_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION", "PURE_FP16"]
+    assert [p.value for p in fo.Precision] == [1, 2, 3, 4]  # auto() values of adam.py:19-23
+    assert issubclass(fo.Adam, torch.optim.Optimizer)
+    assert issubclass(fo.GradScaler, torch.amp.GradScaler)

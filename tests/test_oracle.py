@@ -159,15 +159,21 @@ def test_constant_gradient_closed_form(oracle, eps_mode, bias_correction):
         want_p = want_p - ss * m_t / denom
         assert np.allclose(m, m_t, rtol=5e-6)
         assert np.allclose(v, v_t, rtol=5e-6)
-        assert np.allclose(p - p0, want_p - p0, rtol=2e-5, atol=3e-7 * np.abs(p0).max())
+        # p is rounded to float32 every step: half an ulp of |p| per step on top of the movement's own error
+        assert (np.abs((p - p0) - (want_p - p0)) <= 2e-5 * np.abs(want_p - p0) + t * 1.2e-7 * np.abs(p0) + 1e-9).all()
 
 
 def test_first_step_is_sign_descent(oracle):
-    """m=v=0, wd=0, eps outside: dp = -lr*g/(|g| + eps/sqrt(1-b2)), i.e. -lr*sign(g) for |g| >> eps."""
-    g = np.array([1e-3, -1e-3, 0.5, -7.0], np.float32)
-    p = np.zeros(4, np.float32); m = np.zeros(4, np.float32); v = np.zeros(4, np.float32)
+    """m=v=0, wd=0, eps outside: dp = -lr*g/(|g| + eps/sqrt(1-b2)), i.e. -lr*sign(g) for |g| >> eps/sqrt(1-b2)."""
+    g = np.array([1e-3, -1e-3, 0.5, -7.0, 1e-7], np.float32)
+    p = np.zeros(5, np.float32); m = np.zeros(5, np.float32); v = np.zeros(5, np.float32)
     oracle.step_c(FULL, p, m, v, g, None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1)
-    assert np.allclose(p, -1e-3 * np.sign(g), rtol=1e-4)
+    b2 = float(np.float32(0.999))
+    g64 = g.astype(np.float64)
+    want = -float(np.float32(1e-3)) * g64 / (np.abs(g64) + float(np.float32(1e-8)) / math.sqrt(1 - b2))
+    assert np.allclose(p, want, rtol=2e-6)
+    assert np.allclose(p[2:4], -1e-3 * np.sign(g[2:4]), rtol=1e-5)  # large gradients: plain sign descent
+    assert abs(p[4]) < 0.3e-3  # a gradient of the size of eps/sqrt(1-b2) moves much less than lr
 
 
 def test_zero_gradient_decay_and_weight_decay(oracle):
@@ -470,8 +476,12 @@ def test_torch_cpu_baseline_matches_oracle(oracle, mode):
         kw = dict(HY, grad_scale=gs, optim_scale=65536.0 if mode == PURE16 else 1.0, decay=0.01, step=step)
         oracle.step_c(mode, t.p[0], t.m[0], t.v[0], g, t.p16[0] if t.p16 else None, **kw)
         step_torch_cpu(mode, tp, tm, tv, torch.from_numpy(g), tpc, **kw)
+    # a timing baseline, not a checker: torch's fused CPU loops round differently in the last place
     for got, want in ((tp, t.p[0]), (tm, t.m[0]), (tv, t.v[0])):
+        scale = float(np.abs(want.astype(np.float32)).max())
+        diff = np.abs(got.numpy().astype(np.float32) - want.astype(np.float32))
         if want.dtype == np.float16:
-            assert C.ulp_distance_f16(got.numpy(), want).max() <= 2
+            ok = (C.ulp_distance_f16(got.numpy(), want) <= 2) | (diff <= 1e-4 * scale)
         else:
-            assert np.allclose(got.numpy(), want, rtol=1e-5, atol=1e-10)
+            ok = diff <= 1e-5 * np.abs(want) + 1e-5 * scale
+        assert ok.all()
