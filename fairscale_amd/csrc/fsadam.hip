@@ -337,8 +337,8 @@ struct Options {
 int64_t default_lds_throttle(int mode) {
     switch (mode) {
         case FSADAM_FULL_PRECISION: return 16384;
-        case FSADAM_MIXED_PRECISION: return 16384;
-        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 13312;
+        case FSADAM_MIXED_PRECISION: return 15360;
+        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
         default: return 13312;
     }
 }

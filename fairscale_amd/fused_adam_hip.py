@@ -89,9 +89,10 @@ def rows_of_lists(tensor_lists: Sequence[Sequence[torch.Tensor]]) -> np.ndarray:
     """(n, 6) int64: p, m, v, g, p_copy pointers and numel -- the memory layout of FsAdamTensor[n]."""
     n = len(tensor_lists[0])
     rows = np.zeros((n, _ROW_WORDS), dtype=np.int64)
+    data_ptr, numel = torch.Tensor.data_ptr, torch.Tensor.numel
     for d, lst in enumerate(tensor_lists):
-        rows[:, d] = [t.data_ptr() for t in lst]
-    rows[:, 5] = [t.numel() for t in tensor_lists[0]]
+        rows[:, d] = list(map(data_ptr, lst))  # C-level loop: this runs every step for every tensor
+    rows[:, 5] = list(map(numel, tensor_lists[0]))
     return rows
 
 

@@ -52,19 +52,6 @@ _NATIVE_MODE = {
 _MAX_OPTIM_SCALE = 2 ** 16
 
 
-class _DeviceBatch:
-    """The tensor lists of one param group on one device, in the order the native call wants them."""
-
-    __slots__ = ("lists",)
-
-    def __init__(self, depth: int):
-        self.lists: List[List[torch.Tensor]] = [[] for _ in range(depth)]
-
-    def add(self, tensors: Tuple[torch.Tensor, ...]) -> None:
-        for lst, t in zip(self.lists, tensors):
-            lst.append(t)
-
-
 class Adam(torch.optim.Optimizer):
     """Fused Adam on MI355X. GPU-only.
 
@@ -195,6 +182,7 @@ class Adam(torch.optim.Optimizer):
         for plan in self.__dict__.get("_plans", {}).values():
             plan.close()
         self._plans = {}
+        self._group_cache = {}
 
     def _flag_for(self, device: torch.device) -> torch.Tensor:
         flag = self._flags.get(device)
@@ -202,6 +190,76 @@ class Adam(torch.optim.Optimizer):
             flag = torch.zeros(1, dtype=torch.float32, device=device)
             self._flags[device] = flag
         return flag
+
+    def _gather(self, gi: int, group: Dict[str, Any]):
+        """The per-parameter walk of adam.py:207-254: lazy state, step counters, tensor lists per device.
+        Also (re)builds the group's fast-path cache when every parameter took part and shares one device."""
+        mixed = self.mixed_precision
+        state_map, optim_type = self.state, self.optim_type
+        masters = self.fp32_param_groups[gi]["params"] if mixed else None
+        batches: Dict[torch.device, List[List[torch.Tensor]]] = {}
+        states: List[dict] = []
+        step_no = None
+        params = group["params"]
+        for pj, p in enumerate(params):
+            grad = p.grad
+            if grad is None:
+                continue
+            if grad.is_sparse:
+                raise RuntimeError("FusedAdam does not support sparse gradients, please consider SparseAdam instead")
+            state = state_map[p]
+            if len(state) == 0:  # adam.py:223-228
+                state["step"] = 0
+                state["exp_avg"] = torch.zeros_like(p, dtype=optim_type)
+                state["exp_avg_sq"] = torch.zeros_like(p, dtype=optim_type)
+            step_no = state["step"] = state["step"] + 1  # the call uses the last parameter's counter (adam.py:272)
+            states.append(state)
+            lists = batches.get(p.device)
+            if lists is None:
+                lists = batches[p.device] = [[] for _ in range(5 if mixed else 4)]
+            lists[0].append(masters[pj] if mixed else p)
+            lists[1].append(state["exp_avg"])
+            lists[2].append(state["exp_avg_sq"])
+            lists[3].append(grad)
+            if mixed:
+                lists[4].append(p)
+        caches = self.__dict__.setdefault("_group_cache", {})
+        if len(states) == len(params) and len(batches) == 1:
+            device = next(iter(batches))
+            caches[gi] = (params, len(params), states, masters, device)
+        else:
+            caches.pop(gi, None)
+        return batches, step_no
+
+    def _gather_fast(self, gi: int, group: Dict[str, Any]):
+        """Same result as ``_gather`` for the steady state (every parameter of the group has a dense
+        gradient and an initialised state, all on one device) without the per-parameter dictionary
+        walk; returns (None, None) when that does not hold and the general walk must run."""
+        cache = self.__dict__.get("_group_cache", {}).get(gi)
+        if cache is None:
+            return None, None
+        params, count, states, masters, device = cache
+        if group["params"] is not params or len(params) != count or count == 0:
+            return None, None
+        if self.state.get(params[-1]) is not states[-1] or self.state.get(params[0]) is not states[0]:
+            return None, None  # the state mapping was replaced (e.g. load_state_dict)
+        if masters is not None and (self.fp32_param_groups[gi]["params"] is not masters or len(masters) != count):
+            return None, None  # the fp32 master copies were rebuilt or replaced
+        grads = [p.grad for p in params]
+        for g in grads:
+            if g is None or g.is_sparse:
+                return None, None
+        try:
+            m_list = [st["exp_avg"] for st in states]
+            v_list = [st["exp_avg_sq"] for st in states]
+        except KeyError:  # a state dict was emptied behind our back: let the general walk re-initialise it
+            return None, None
+        for st in states:
+            st["step"] += 1
+        lists = [masters if masters is not None else params, m_list, v_list, grads]
+        if masters is not None:
+            lists.append(params)
+        return {device: lists}, states[-1]["step"]
 
     def step(self, closure: Optional[Callable[[], float]] = None, *, scale: float = 1.0) -> Optional[float]:
         """One optimization step (adam.py:184-297).
@@ -214,41 +272,19 @@ class Adam(torch.optim.Optimizer):
         self.__dict__.setdefault("_plans", {})  # absent after unpickling
         self.__dict__.setdefault("_flags", {})
         native_mode = _NATIVE_MODE[self.precision]
-        mixed = self.mixed_precision
         watch_overflow = self.precision is Precision.PURE_FP16
 
         for gi, group in enumerate(self.param_groups):
-            batches: Dict[torch.device, _DeviceBatch] = {}
             beta1, beta2 = group["betas"]
-            step_no = None
-            for pj, p in enumerate(group["params"]):
-                if p.grad is None:
-                    continue
-                grad = p.grad.data
-                if grad.is_sparse:
-                    raise RuntimeError("FusedAdam does not support sparse gradients, please consider SparseAdam instead")
-                state = self.state[p]
-                if len(state) == 0:  # adam.py:223-228
-                    state["step"] = 0
-                    state["exp_avg"] = torch.zeros_like(p, dtype=self.optim_type)
-                    state["exp_avg_sq"] = torch.zeros_like(p, dtype=self.optim_type)
-                state["step"] += 1
-                step_no = state["step"]  # the call uses the last parameter's counter (adam.py:272)
-                batch = batches.get(p.device)
-                if batch is None:
-                    batch = batches[p.device] = _DeviceBatch(5 if mixed else 4)
-                if mixed:
-                    master = self.fp32_param_groups[gi]["params"][pj]
-                    batch.add((master.data, state["exp_avg"], state["exp_avg_sq"], grad, p.data))
-                else:
-                    batch.add((p.data, state["exp_avg"], state["exp_avg_sq"], grad))
-
+            batches, step_no = self._gather_fast(gi, group)
+            if batches is None:
+                batches, step_no = self._gather(gi, group)
             if not batches:
                 # adam.py:256 indexes the first device of an empty dict
                 raise IndexError("list index out of range")
 
             flags: List[torch.Tensor] = []
-            for device, batch in batches.items():
+            for device, lists in batches.items():
                 flag = None
                 if watch_overflow:
                     flag = self._flag_for(device)
@@ -257,7 +293,7 @@ class Adam(torch.optim.Optimizer):
                 plan = self._plans.get((gi, device))
                 if plan is None:
                     plan = self._plans[(gi, device)] = TensorListPlan(native_mode, device)
-                plan.step(batch.lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
+                plan.step(lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
                           step_no, self.eps_mode, 1 if group["bias_correction"] else 0, group["weight_decay"])
 
             overflowed = bool(sum(f.item() for f in flags)) if flags else False  # adam.py:278
