@@ -443,29 +443,44 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
 
 }  // namespace
 
+// A device table plus its pinned staging copy.  A plan keeps a small ring of them: when a pointer
+// of the list moves, the new table goes into the next slot, so the host only ever waits for the
+// step that used that slot kTableSlots updates ago, not for the step still in flight.
+struct TableSlot {
+    int64_t cap_descs = 0;
+    ChunkDesc* d_table = nullptr;
+    ChunkDesc* h_table = nullptr;  // pinned
+    hipEvent_t last_use = nullptr;
+    bool used = false;
+};
+constexpr int kTableSlots = 3;
+
 struct FsAdamPlan {
     int mode = 0;
     int device = -1;
     Options opt;
     Layout layout;
-    std::vector<FsAdamTensor> rows;  // what the device table was built from
+    std::vector<FsAdamTensor> rows;  // what the current table was built from
     int64_t uploads = 0;
-    int64_t cap_descs = 0;  // capacity of d_table / h_table, in descriptors
-    ChunkDesc* d_table = nullptr;
-    ChunkDesc* h_table = nullptr;  // pinned staging
-    hipEvent_t last_use = nullptr;
-    bool used = false;
+    TableSlot slots[kTableSlots];
+    int current = -1;  // slot holding the table of `rows`
     uint64_t lru = 0;  // fsadam_step cache bookkeeping
 };
 
 namespace {
 
+void slot_release(TableSlot& slot) {
+    if (slot.used && slot.last_use) (void)hipEventSynchronize(slot.last_use);
+    if (slot.d_table) (void)hipFree(slot.d_table);
+    if (slot.h_table) (void)hipHostFree(slot.h_table);
+    slot.d_table = slot.h_table = nullptr;
+    slot.cap_descs = 0;
+    slot.used = false;
+}
+
 void plan_release_buffers(FsAdamPlan* plan) {
-    if (plan->used && plan->last_use) (void)hipEventSynchronize(plan->last_use);
-    if (plan->d_table) (void)hipFree(plan->d_table);
-    if (plan->h_table) (void)hipHostFree(plan->h_table);
-    plan->d_table = plan->h_table = nullptr;
-    plan->cap_descs = 0;
+    for (TableSlot& slot : plan->slots) slot_release(slot);
+    plan->current = -1;
 }
 
 char* advance(const void* base, int64_t elems, int elem_size) {
@@ -534,7 +549,6 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     if (plan->device != dev) {
         plan_release_buffers(plan);
         plan->device = dev;
-        if (!plan->last_use) FS_HIP(hipEventCreateWithFlags(&plan->last_use, hipEventDisableTiming));
     }
     {
         std::lock_guard<std::mutex> lock(g_mutex);
@@ -546,25 +560,27 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     if (L.n_large_descs * (L.large_chunk_elems / L.tile_elems) > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0)
         return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
-    // the previous table may still be read by a kernel in flight
-    if (plan->used) FS_HIP(hipEventSynchronize(plan->last_use));
-    if (n_descs > plan->cap_descs) {
-        plan_release_buffers(plan);
+    // next slot of the ring; it may still be read by the step that used it last
+    TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
+    if (!slot.last_use) FS_HIP(hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming));
+    if (slot.used) FS_HIP(hipEventSynchronize(slot.last_use));
+    if (n_descs > slot.cap_descs) {
+        slot_release(slot);
         const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
-        if (hipMalloc(reinterpret_cast<void**>(&plan->d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
-            plan->d_table = nullptr;
+        if (hipMalloc(reinterpret_cast<void**>(&slot.d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
+            slot.d_table = nullptr;
             return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
         }
-        if (hipHostMalloc(reinterpret_cast<void**>(&plan->h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
-            (void)hipFree(plan->d_table);
-            plan->d_table = plan->h_table = nullptr;
+        if (hipHostMalloc(reinterpret_cast<void**>(&slot.h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
+            (void)hipFree(slot.d_table);
+            slot.d_table = slot.h_table = nullptr;
             return fail(FSADAM_ENOMEM, "hipHostMalloc of the descriptor staging buffer failed");
         }
-        plan->cap_descs = cap;
+        slot.cap_descs = cap;
     }
     // large tensors first (one launch), then small ones (second launch)
-    ChunkDesc* large = plan->h_table;
-    ChunkDesc* small = plan->h_table + L.n_large_descs;
+    ChunkDesc* large = slot.h_table;
+    ChunkDesc* small = slot.h_table + L.n_large_descs;
     for (int64_t t = 0; t < n; ++t) {
         const FsAdamTensor& r = tensors[t];
         if (r.numel == 0) continue;
@@ -580,16 +596,17 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     plan->layout = L;
     plan->rows.assign(tensors, tensors + n);
     if (n_descs > 0)
-        FS_HIP(hipMemcpyAsync(plan->d_table, plan->h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
-    FS_HIP(hipEventRecord(plan->last_use, stream));
-    plan->used = true;
+        FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
+    FS_HIP(hipEventRecord(slot.last_use, stream));
+    slot.used = true;
+    plan->current = (plan->current + 1) % kTableSlots;
     plan->uploads += 1;
     return FSADAM_OK;
 }
 
 int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, float grad_scale, float optim_scale,
               float decay, int step, int eps_mode, int bias_correction, float* found_inf, hipStream_t stream) {
-    if (plan->rows.empty()) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
+    if (plan->rows.empty() || plan->current < 0) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
     if (eps_mode != FSADAM_EPS_INSIDE_SQRT && eps_mode != FSADAM_EPS_OUTSIDE_SQRT)
         return fail(FSADAM_EINVAL, "eps_mode must be 0 (inside sqrt) or 1 (outside)");
     if (plan->mode == FSADAM_PURE_FP16 && !found_inf) return fail(FSADAM_EINVAL, "PURE_FP16 needs a found_inf device pointer");
@@ -613,11 +630,12 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
 
     const Layout& L = plan->layout;
     const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
-    int rc = launch_mode(plan->mode, plan->d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
+    TableSlot& slot = plan->slots[plan->current];
+    int rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
     if (rc) return rc;
-    rc = launch_mode(plan->mode, plan->d_table + L.n_large_descs, L.n_small_descs, 0, plan->opt, s, found_inf, stream);
+    rc = launch_mode(plan->mode, slot.d_table + L.n_large_descs, L.n_small_descs, 0, plan->opt, s, found_inf, stream);
     if (rc) return rc;
-    FS_HIP(hipEventRecord(plan->last_use, stream));
+    FS_HIP(hipEventRecord(slot.last_use, stream));
     return FSADAM_OK;
 }
 
@@ -767,7 +785,8 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
 int fsadam_plan_destroy(FsAdamPlan* plan) {
     if (!plan) return FSADAM_OK;
     plan_release_buffers(plan);
-    if (plan->last_use) (void)hipEventDestroy(plan->last_use);
+    for (TableSlot& slot : plan->slots)
+        if (slot.last_use) (void)hipEventDestroy(slot.last_use);
     delete plan;
     return FSADAM_OK;
 }

@@ -133,7 +133,11 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
                 int eps_mode, int bias_correction, float* found_inf_dev, void* hip_stream);
 
 /* ---- explicit plans: same step, table lifetime owned by the caller (what the Python optimizer
- * uses so that an OSS/FSDP shard's table is built once and re-sent only when a pointer moves). */
+ * uses so that an OSS/FSDP shard's table is built once and re-sent only when a pointer moves).
+ * A plan belongs to the device that was current at its first fsadam_plan_set_tensors and must not
+ * be used by two threads at once.  fsadam_plan_set_tensors may be called while earlier steps of the
+ * plan are still running: tables rotate through a ring of three, and the call only waits for the
+ * step that last used the slot it is about to overwrite. */
 int fsadam_plan_create(int precision_mode, FsAdamPlan** out);
 int fsadam_plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n_tensors, void* hip_stream);
 int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, float grad_scale,
