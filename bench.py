@@ -104,6 +104,31 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
     return out
 
 
+def measure_grad_pass(torch, numel, steps, warmup, device):
+    """The pre-step gradient pass over the same shard's fp16 gradients: norms + overflow check only
+    (2 B/param read) and with the unscale written back (2 B read + 2 B written)."""
+    from fairscale_amd.grad_pass import grad_pass
+
+    g = torch.empty(numel, device=device, dtype=torch.float16).normal_(0, 1.0)
+    out = {}
+    for name, write_back, bpp in (("norm_and_check", False, 2), ("unscale_norm_and_check", True, 4)):
+        inv = 1.0 / 1024 if not write_back else 1.0 - 2.0 ** -12  # written back every step: keep the values in range
+        for _ in range(warmup):
+            grad_pass([g], inv, write_back=write_back)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            grad_pass([g], inv, write_back=write_back)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        out[name] = {"ms": ms, "bytes_per_param": bpp, "achieved_gbs": numel * bpp / ms / 1e6, "frac_of_hbm_peak": numel * bpp / ms / 1e6 / HBM_PEAK_GBS}
+    del g
+    torch.cuda.empty_cache()
+    return out
+
+
 def measure_cpu(torch, precision_name, numel, budget_s=15.0):
     """The same math as in-place torch CPU ops on `numel` parameters; stops after ~budget_s."""
     from oracle import adam_oracle as O
@@ -178,6 +203,8 @@ def main():
         r = measure_gpu(torch, "MIXED_PRECISION", args.numel, args.steps, args.warmup, device)
         also["MIXED_PRECISION"] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
                                    "achieved_gbs": r["achieved_gbs"], "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
+    if not args.no_also:
+        also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"

@@ -37,6 +37,14 @@ class _Int64Fields(ctypes.Structure):
         return {name: int(getattr(self, name)) for name, _ in self._fields_}
 
 
+class FsGradTensor(ctypes.Structure):
+    _fields_ = [("g", ctypes.c_void_p), ("numel", ctypes.c_int64)]
+
+
+GRAD_F32 = 0
+GRAD_F16 = 1
+
+
 class FsAdamPlanInfo(_Int64Fields):
     _fields_ = [("mode", ctypes.c_int32), ("device", ctypes.c_int32)] + [
         (name, ctypes.c_int64)
@@ -69,6 +77,7 @@ SIGNATURES = {
     "fsadam_plan_info": (_i32, [_vp, ctypes.POINTER(FsAdamPlanInfo)]),
     "fsadam_plan_destroy": (_i32, [_vp]),
     "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),
+    "fsadam_grad_pass": (_i32, [ctypes.POINTER(FsGradTensor), _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _vp]),
     "fsadam_clear_cache": (_i32, []),
     "fsadam_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
 }

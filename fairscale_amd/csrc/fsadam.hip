@@ -134,9 +134,10 @@ __device__ __forceinline__ void store_vec(gptr<T> ptr, typename VecOf<T, E>::typ
 
 // Two packed halves in one 32-bit word: non-zero when either is +-inf or NaN (exponent field all
 // ones).  Adding 0x0400 to an all-ones exponent field carries into the sign position; any smaller
-// field does not, and the low half cannot carry into the high one.  The test is kept in integer
-// arithmetic on whole words on purpose: written as per-element comparisons OR-ed into a bool, the
-// compiler's vectorised form only looked at the first element of each packet.
+// field does not, and the low half cannot carry into the high one.  Whole words, three integer
+// operations per two halves.  (A per-element form, __builtin_bit_cast(uint16_t, h[e]) on the elements
+// of a half vector, silently tested element 0 eight times: this compiler's bit_cast of a vector
+// ELEMENT always reads element 0.  Bit-cast whole vectors, or copy the element to a scalar first.)
 __device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w) {
     return ((w & 0x7c007c00u) + 0x04000400u) & 0x80008000u;
 }
@@ -293,6 +294,227 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
     }
     // Same-value store from every lane that stored a non-finite fp16 m or v (kernel.cu:103-105).
     if (ModeTraits<MODE>::kScaled && bad != 0) *(gptr<float>)found_inf = 1.0f;
+}
+
+
+// --------------------------------------------------------------------------------------------
+// gradient pass: non-finite check + unscale + sum of squares + max |g| in ONE read of the gradients
+// (what torch._amp_foreach_non_finite_check_and_unscale_, called from
+// fairscale/optim/grad_scaler.py:211-215, and calc_grad_norm, fairscale/internal/params.py:59-76,
+// do in two or more passes)
+// --------------------------------------------------------------------------------------------
+
+template <typename T>
+struct GradTraits;
+template <>
+struct GradTraits<float> { static constexpr int kElems = 4; };
+template <>
+struct GradTraits<_Float16> { static constexpr int kElems = 8; };
+
+// Magnitudes are compared as integers: with the sign bit cleared, IEEE bit patterns order like the
+// values, +inf is the largest finite-exponent pattern and every NaN is larger still.  One unsigned
+// maximum therefore gives the max norm (a NaN wins, as in torch's abs().max()) and, taken over the
+// incoming values, the overflow check (maximum >= the pattern of +inf) -- no floating compare, no
+// per-element branch.  For halves two magnitudes travel in one 32-bit word (packed u16 maximum).
+struct GradPartial {  // one per workgroup, written unconditionally
+    double sum_squares;
+    uint32_t stored_max;    // largest magnitude pattern of the values unscaling stores
+    uint32_t incoming_max;  // largest magnitude pattern of the gradients as read
+};
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t max_u16x2(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+
+// How the stored value r is formed from g: as is; by a packed half multiply (exact product, one
+// rounding: the same bits as float(g) * inv_scale rounded to half whenever inv_scale is itself a
+// half); or through float.
+enum : int { kGradUnit = 0, kGradHalfScale = 1, kGradFloatScale = 2 };
+
+struct GradAcc {
+    float sum = 0.f;
+    uint32_t stored_max = 0;
+    uint32_t incoming_max = 0;
+};
+
+// two halves in one word
+template <int HOW>
+__device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2 inv_half, GradAcc& acc) {
+    acc.incoming_max = max_u16x2(acc.incoming_max, w & 0x7fff7fffu);
+    f16x2 r = __builtin_bit_cast(f16x2, w);
+    if (HOW == kGradHalfScale) {
+        r = r * inv_half;
+    } else if (HOW == kGradFloatScale) {
+        r[0] = (_Float16)((float)r[0] * inv_scale);
+        r[1] = (_Float16)((float)r[1] * inv_scale);
+    }
+    const uint32_t out = __builtin_bit_cast(uint32_t, r);
+    if (HOW != kGradUnit) acc.stored_max = max_u16x2(acc.stored_max, out & 0x7fff7fffu);
+    // fused multiply-adds with half operands widened on the fly (v_fma_mix_f32): the product of two
+    // halves is exact in fp32, subnormal halves included
+    acc.sum = __builtin_fmaf((float)r[0], (float)r[0], acc.sum);
+    acc.sum = __builtin_fmaf((float)r[1], (float)r[1], acc.sum);
+    return out;
+}
+
+__device__ __forceinline__ _Float16 grad_scalar(_Float16 g, int how, float inv_scale, GradAcc& acc) {
+    const uint32_t w = __builtin_bit_cast(uint16_t, g);
+    uint32_t out;
+    if (how == kGradUnit) out = grad_word<kGradUnit>(w, inv_scale, f16x2{}, acc);
+    else out = grad_word<kGradFloatScale>(w, inv_scale, f16x2{}, acc);  // the two scaled forms give the same bits
+    return __builtin_bit_cast(_Float16, (uint16_t)out);
+}
+
+template <int HOW>
+__device__ __forceinline__ float grad_float(float g, float inv_scale, GradAcc& acc) {
+    const uint32_t mag = __builtin_bit_cast(uint32_t, g) & 0x7fffffffu;
+    acc.incoming_max = mag > acc.incoming_max ? mag : acc.incoming_max;
+    const float r = (HOW == kGradUnit) ? g : g * inv_scale;
+    if (HOW != kGradUnit) {
+        const uint32_t rm = __builtin_bit_cast(uint32_t, r) & 0x7fffffffu;
+        acc.stored_max = rm > acc.stored_max ? rm : acc.stored_max;
+    }
+    acc.sum += r * r;
+    return r;
+}
+
+__device__ __forceinline__ float grad_scalar(float g, int how, float inv_scale, GradAcc& acc) {
+    return how == kGradUnit ? grad_float<kGradUnit>(g, inv_scale, acc) : grad_float<kGradFloatScale>(g, inv_scale, acc);
+}
+
+template <typename T, int BLOCK, int ITEMS, int HOW, bool WRITE>
+__device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, float inv_scale, GradAcc& acc) {
+    constexpr int E = GradTraits<T>::kElems;
+    constexpr uint32_t kTile = BLOCK * E * ITEMS;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint32_t left = d.n - off;
+    gptr<T> g = (gptr<T>)const_cast<void*>(d.g) + off;
+    if (d.vector_ok && left >= kTile) {
+        u32x4 raw[ITEMS];
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4>>(g + (k * BLOCK + threadIdx.x) * E));
+        const f16x2 inv_half = {(_Float16)inv_scale, (_Float16)inv_scale};
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // NB: copy the element out before __builtin_bit_cast: applied directly to a vector
+                // element (bit_cast(T, v[e])) this compiler reads element 0 whatever e is.
+                const uint32_t word = raw[k][e];
+                if constexpr (sizeof(T) == 2) raw[k][e] = grad_word<HOW>(word, inv_scale, inv_half, acc);
+                else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
+            }
+            if (WRITE && HOW != kGradUnit)
+                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4>>(g + (k * BLOCK + threadIdx.x) * E));
+        }
+    } else {
+        const uint32_t count = left < kTile ? left : kTile;
+        for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
+            const T r = grad_scalar(g[e], HOW, inv_scale, acc);
+            if (WRITE && HOW != kGradUnit) g[e] = r;
+        }
+    }
+}
+
+template <typename T, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, float inv_scale_value,
+                                                           const float* __restrict__ inv_scale_dev, int write_back,
+                                                           GradPartial* __restrict__ partials) {
+    static_assert(BLOCK == 64, "one wave per workgroup: the partial is reduced with wave shuffles only");
+    constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
+    const uint32_t block = blockIdx.x;
+    const uint32_t chunk = block >> log2k;
+    const uint32_t off = (block & ((1u << log2k) - 1u)) * kTile;
+    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
+    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
+        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
+    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    // the scale may live on the device (a loss scaler keeps it there): uniform address, scalar load
+    const float inv_scale = inv_scale_dev ? *(const __attribute__((address_space(4))) float*)inv_scale_dev : inv_scale_value;
+
+    GradAcc acc;
+    if (off < d.n) {
+        if (inv_scale == 1.0f) {
+            grad_tile<T, BLOCK, ITEMS, kGradUnit, false>(d, off, inv_scale, acc);
+        } else if (sizeof(T) == 2 && (float)(_Float16)inv_scale == inv_scale) {
+            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradHalfScale, true>(d, off, inv_scale, acc);
+            else grad_tile<T, BLOCK, ITEMS, kGradHalfScale, false>(d, off, inv_scale, acc);
+        } else {
+            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradFloatScale, true>(d, off, inv_scale, acc);
+            else grad_tile<T, BLOCK, ITEMS, kGradFloatScale, false>(d, off, inv_scale, acc);
+        }
+        if (inv_scale == 1.0f) acc.stored_max = acc.incoming_max;  // nothing was rescaled
+    }
+    if (sizeof(T) == 2) {  // unpack the two 16-bit maxima
+        acc.stored_max = (acc.stored_max & 0xffffu) > (acc.stored_max >> 16) ? (acc.stored_max & 0xffffu) : (acc.stored_max >> 16);
+        acc.incoming_max = (acc.incoming_max & 0xffffu) > (acc.incoming_max >> 16) ? (acc.incoming_max & 0xffffu) : (acc.incoming_max >> 16);
+    }
+    // wave reduction in a fixed order (xor butterfly): the same inputs always give the same bits
+    double dsum = (double)acc.sum;
+    uint32_t smax = acc.stored_max, imax = acc.incoming_max;
+#pragma unroll
+    for (int w = 32; w >= 1; w >>= 1) {
+        dsum += __shfl_xor(dsum, w, 64);
+        const uint32_t s2 = (uint32_t)__shfl_xor((int)smax, w, 64), i2 = (uint32_t)__shfl_xor((int)imax, w, 64);
+        smax = s2 > smax ? s2 : smax;
+        imax = i2 > imax ? i2 : imax;
+    }
+    if (threadIdx.x == 0) {
+        gptr<GradPartial> out = (gptr<GradPartial>)partials + block;
+        out->sum_squares = dsum;
+        out->stored_max = smax;
+        out->incoming_max = imax;
+    }
+}
+
+// Fixed-order reduction of `n` partials into `out[blockIdx.x]`: block b takes the b-th contiguous
+// slice, thread t every 256th entry of it, then a shared-memory tree.
+__global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
+                                                          GradPartial* __restrict__ out) {
+    __shared__ double s_sum[256];
+    __shared__ uint32_t s_stored[256];
+    __shared__ uint32_t s_incoming[256];
+    const uint32_t lo = blockIdx.x * per_block;
+    const uint32_t hi = lo + per_block < n ? lo + per_block : n;
+    double sum = 0.0;
+    uint32_t stored = 0, incoming = 0;
+    for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+        const GradPartial p = in[i];
+        sum += p.sum_squares;
+        stored = p.stored_max > stored ? p.stored_max : stored;
+        incoming = p.incoming_max > incoming ? p.incoming_max : incoming;
+    }
+    s_sum[threadIdx.x] = sum; s_stored[threadIdx.x] = stored; s_incoming[threadIdx.x] = incoming;
+    __syncthreads();
+    for (int w = 128; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+            s_stored[threadIdx.x] = s_stored[threadIdx.x + w] > s_stored[threadIdx.x] ? s_stored[threadIdx.x + w] : s_stored[threadIdx.x];
+            s_incoming[threadIdx.x] = s_incoming[threadIdx.x + w] > s_incoming[threadIdx.x] ? s_incoming[threadIdx.x + w] : s_incoming[threadIdx.x];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        out[blockIdx.x].sum_squares = s_sum[0];
+        out[blockIdx.x].stored_max = s_stored[0];
+        out[blockIdx.x].incoming_max = s_incoming[0];
+    }
+}
+
+// Hands the single remaining partial to the caller's three outputs.
+__global__ void fsadam_grad_publish(const GradPartial* __restrict__ total, int is_half, float* found_inf, double* sum_squares,
+                                    float* abs_max) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
+        if (total->incoming_max >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
+        if (sum_squares) *sum_squares = total->sum_squares;
+        if (abs_max)
+            *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)total->stored_max) : __builtin_bit_cast(float, total->stored_max);
+    }
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -639,6 +861,174 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     return FSADAM_OK;
 }
 
+
+// ---- gradient pass, host side -----------------------------------------------------------------
+
+struct GradPlan {
+    int device = -1;
+    int dtype = 0;
+    std::vector<FsGradTensor> rows;
+    Layout layout;
+    TableSlot slots[kTableSlots];
+    int current = -1;
+    GradPartial* d_partials = nullptr;  // [cap_partials] first stage, then [kReduceBlocks] second stage, then [1] total
+    int64_t cap_partials = 0;
+    hipEvent_t last_use = nullptr;
+    bool used = false;
+    uint64_t lru = 0;
+};
+
+constexpr int kGradItems = 4;        // 16-byte vectors per lane: 4 KiB per wave
+constexpr int kGradThrottle = 13312; // LDS ballast per workgroup for the gradient kernels
+constexpr int kReduceBlocks = 512;
+
+int grad_elem_size(int dtype) { return dtype == FSADAM_GRAD_F16 ? 2 : 4; }
+int64_t grad_tile_elems(int dtype) { return 64 * (16 / grad_elem_size(dtype)) * kGradItems; }
+
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype) {
+    Layout L;
+    L.tile_elems = grad_tile_elems(dtype);
+    int64_t min_large = 0;
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t numel = grads[t].numel;
+        L.total_elems += numel;
+        if (numel == 0) { L.n_empty += 1; continue; }
+        (aligned_to(grads[t].g, 16) ? L.n_vector : L.n_scalar) += 1;
+        if (numel >= kLargeThreshold) {
+            L.n_large += 1;
+            if (min_large == 0 || numel < min_large) min_large = numel;
+        } else {
+            L.n_small += 1;
+        }
+    }
+    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t numel = grads[t].numel;
+        if (numel == 0) continue;
+        if (numel >= kLargeThreshold) L.n_large_descs += ceil_div(numel, L.large_chunk_elems);
+        else L.n_small_descs += ceil_div(numel, L.tile_elems);
+    }
+    return L;
+}
+
+void grad_plan_free(GradPlan* plan) {
+    if (plan->used && plan->last_use) (void)hipEventSynchronize(plan->last_use);
+    for (TableSlot& slot : plan->slots) {
+        slot_release(slot);
+        if (slot.last_use) (void)hipEventDestroy(slot.last_use);
+    }
+    if (plan->d_partials) (void)hipFree(plan->d_partials);
+    if (plan->last_use) (void)hipEventDestroy(plan->last_use);
+    delete plan;
+}
+
+int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
+    const Layout L = grad_layout(grads, n, plan->dtype);
+    const int64_t k = L.large_chunk_elems / L.tile_elems;
+    const int64_t n_blocks = L.n_large_descs * k + L.n_small_descs;
+    if (L.n_large_descs * k > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
+    const int64_t n_descs = L.n_large_descs + L.n_small_descs;
+    TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
+    if (!slot.last_use) FS_HIP(hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming));
+    if (!plan->last_use) FS_HIP(hipEventCreateWithFlags(&plan->last_use, hipEventDisableTiming));
+    if (slot.used) FS_HIP(hipEventSynchronize(slot.last_use));
+    if (n_descs > slot.cap_descs) {
+        slot_release(slot);
+        const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
+        if (hipMalloc(reinterpret_cast<void**>(&slot.d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
+            slot.d_table = nullptr;
+            return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
+        }
+        if (hipHostMalloc(reinterpret_cast<void**>(&slot.h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
+            (void)hipFree(slot.d_table);
+            slot.d_table = slot.h_table = nullptr;
+            return fail(FSADAM_ENOMEM, "hipHostMalloc of the descriptor staging buffer failed");
+        }
+        slot.cap_descs = cap;
+    }
+    if (n_blocks + kReduceBlocks + 1 > plan->cap_partials) {
+        // the partials may still be read by the reduction of the previous call
+        if (plan->used) FS_HIP(hipEventSynchronize(plan->last_use));
+        if (plan->d_partials) (void)hipFree(plan->d_partials);
+        plan->d_partials = nullptr;
+        plan->cap_partials = 0;
+        const int64_t cap = n_blocks + n_blocks / 8 + kReduceBlocks + 1;
+        if (hipMalloc(reinterpret_cast<void**>(&plan->d_partials), cap * sizeof(GradPartial)) != hipSuccess) {
+            plan->d_partials = nullptr;
+            return fail(FSADAM_ENOMEM, "hipMalloc of the partial sums failed");
+        }
+        plan->cap_partials = cap;
+    }
+    const int esz = grad_elem_size(plan->dtype);
+    ChunkDesc* large = slot.h_table;
+    ChunkDesc* small = slot.h_table + L.n_large_descs;
+    for (int64_t t = 0; t < n; ++t) {
+        const FsGradTensor& r = grads[t];
+        if (r.numel == 0) continue;
+        const bool is_large = r.numel >= kLargeThreshold;
+        const int64_t chunk_elems = is_large ? L.large_chunk_elems : L.tile_elems;
+        const int64_t chunks = ceil_div(r.numel, chunk_elems);
+        ChunkDesc*& out = is_large ? large : small;
+        for (int64_t c = 0; c < chunks; ++c) {
+            ChunkDesc& d = out[c];
+            std::memset(&d, 0, sizeof(d));
+            d.g = advance(r.g, c * chunk_elems, esz);
+            d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - c * chunk_elems);
+            d.vector_ok = aligned_to(r.g, 16) ? 1u : 0u;
+        }
+        out += chunks;
+    }
+    plan->layout = L;
+    plan->rows.assign(grads, grads + n);
+    if (n_descs > 0)
+        FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
+    FS_HIP(hipEventRecord(slot.last_use, stream));
+    slot.used = true;
+    plan->current = (plan->current + 1) % kTableSlots;
+    return FSADAM_OK;
+}
+
+template <typename T>
+int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, int write_back, float* found_inf, double* sum_squares,
+                  float* abs_max, hipStream_t stream) {
+    const Layout& L = plan->layout;
+    const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
+    const int64_t large_blocks = L.n_large_descs << log2k;
+    const int64_t n_blocks = large_blocks + L.n_small_descs;
+    TableSlot& slot = plan->slots[plan->current];
+    GradPartial* first = plan->d_partials;
+    GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
+    GradPartial* total = second + kReduceBlocks;
+    if (large_blocks > 0)
+        hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, kGradItems>), dim3((uint32_t)large_blocks), dim3(64), kGradThrottle, stream,
+                           slot.d_table, (uint32_t)log2k, inv_scale, inv_scale_dev, write_back, first);
+    if (L.n_small_descs > 0)
+        hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, kGradItems>), dim3((uint32_t)L.n_small_descs), dim3(64), kGradThrottle, stream,
+                           slot.d_table + L.n_large_descs, 0u, inv_scale, inv_scale_dev, write_back, first + large_blocks);
+    FS_HIP(hipGetLastError());
+    // two fixed-shape reduction steps, then publish (also when the list holds no element: everything is zero)
+    const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_blocks, 1024)));
+    const uint32_t per_block = (uint32_t)ceil_div(std::max<int64_t>(n_blocks, 1), blocks2);
+    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_blocks, per_block, second);
+    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total);
+    hipLaunchKernelGGL(fsadam_grad_publish, dim3(1), dim3(64), 0, stream, total, (int)(sizeof(T) == 2), found_inf, sum_squares, abs_max);
+    FS_HIP(hipGetLastError());
+    FS_HIP(hipEventRecord(slot.last_use, stream));
+    FS_HIP(hipEventRecord(plan->last_use, stream));
+    plan->used = true;
+    return FSADAM_OK;
+}
+
+std::vector<GradPlan*> g_grad_cache;
+constexpr size_t kGradCacheWays = 4;
+
+bool same_grad_rows(const GradPlan* plan, const FsGradTensor* grads, int64_t n) {
+    if ((int64_t)plan->rows.size() != n) return false;
+    for (int64_t t = 0; t < n; ++t)
+        if (plan->rows[t].g != grads[t].g || plan->rows[t].numel != grads[t].numel) return false;
+    return true;
+}
+
 // fsadam_step's table cache
 constexpr size_t kCacheWays = 8;
 std::vector<FsAdamPlan*> g_cache;
@@ -836,10 +1226,60 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
                      found_inf_dev, stream);
 }
 
+
+int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
+                     int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream) {
+    if (grad_dtype != FSADAM_GRAD_F32 && grad_dtype != FSADAM_GRAD_F16) return fail(FSADAM_EINVAL, "unknown gradient dtype " + std::to_string(grad_dtype));
+    if (n_tensors < 1) return fail(FSADAM_EINVAL, "gradient list is empty");
+    if (!grads) return fail(FSADAM_EINVAL, "grads is NULL");
+    for (int64_t t = 0; t < n_tensors; ++t) {
+        if (grads[t].numel < 0) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": negative numel");
+        if (grads[t].numel == 0) continue;
+        if (!grads[t].g) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": NULL pointer");
+        if (!aligned_to(grads[t].g, grad_elem_size(grad_dtype))) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": pointer not aligned to its element size");
+    }
+    int dev = -1;
+    FS_HIP(hipGetDevice(&dev));
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    GradPlan* hit = nullptr;
+    GradPlan* victim = nullptr;
+    for (GradPlan* c : g_grad_cache) {
+        if (c->device == dev && c->dtype == grad_dtype && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+        if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
+    }
+    if (!hit) {
+        if (g_grad_cache.size() < kGradCacheWays || !victim) {
+            GradPlan* fresh = new (std::nothrow) GradPlan();
+            if (!fresh) return fail(FSADAM_ENOMEM, "out of host memory");
+            fresh->device = dev;
+            fresh->dtype = grad_dtype;
+            if (g_grad_cache.size() >= kGradCacheWays) {
+                size_t oldest = 0;
+                for (size_t i = 1; i < g_grad_cache.size(); ++i) if (g_grad_cache[i]->lru < g_grad_cache[oldest]->lru) oldest = i;
+                grad_plan_free(g_grad_cache[oldest]);
+                g_grad_cache[oldest] = fresh;
+            } else {
+                g_grad_cache.push_back(fresh);
+            }
+            victim = fresh;
+        }
+        int rc = grad_plan_set(victim, grads, n_tensors, stream);
+        if (rc) { victim->rows.clear(); return rc; }
+        hit = victim;
+    }
+    hit->lru = ++g_tick;
+    return grad_dtype == FSADAM_GRAD_F16
+               ? grad_plan_run<_Float16>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream)
+               : grad_plan_run<float>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream);
+}
+
 int fsadam_clear_cache(void) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     for (FsAdamPlan* c : g_cache) fsadam_plan_destroy(c);
     g_cache.clear();
+    for (GradPlan* c : g_grad_cache) grad_plan_free(c);
+    g_grad_cache.clear();
     return FSADAM_OK;
 }
 

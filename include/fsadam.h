@@ -152,7 +152,35 @@ int fsadam_plan_destroy(FsAdamPlan* plan);
 int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
                   uint8_t* tensor_class, uint8_t* vector_ok);
 
-/* Drops the tables cached by fsadam_step (synchronises the devices that own them). */
+/* ---- gradient pass: what runs on the gradients BEFORE the step, in one read.
+ * Replaces, for one rank's gradients on one device:
+ *   torch._amp_foreach_non_finite_check_and_unscale_(grads, found_inf, inv_scale)
+ *       as called by fairscale/optim/grad_scaler.py:211-215 (and by torch's GradScaler, which
+ *       fairscale.optim.GradScaler subclasses, grad_scaler.py:60-68), and
+ *   calc_grad_norm(parameters, p) for p = 2 and p = inf, fairscale/internal/params.py:59-76, the
+ *       local norm behind OSS.clip_grad_norm (fairscale/optim/oss.py:244-302) and
+ *       FullyShardedDataParallel.clip_grad_norm_ (fully_sharded_data_parallel.py:621-687).
+ * inv_scale_dev, when not NULL, is a device float[1] that is read instead of the host value inv_scale
+ * (a loss scaler keeps its scale on the device; no host round trip).
+ * Per element: found_inf is raised when the incoming g is +-inf/NaN; r = (inv_scale == 1) ? g :
+ * dtype(float(g) * inv_scale) is what unscaling stores; sum_squares and abs_max are taken of float(r).
+ * write_back != 0 stores r over g (the reference behaviour); write_back == 0 leaves the gradients
+ * untouched, for callers that fold the scale into fsadam_step's grad_scale instead.
+ * Outputs (device pointers, each may be NULL): found_inf_dev float[1], only ever set to 1.0f;
+ * sum_squares_dev double[1] and abs_max_dev float[1], overwritten.  The reductions run in a fixed
+ * order: the same inputs give the same bits.  NaN gradients make both norms NaN, as in torch. */
+typedef struct FsGradTensor {
+    void* g;
+    int64_t numel;
+} FsGradTensor;
+
+#define FSADAM_GRAD_F32 0
+#define FSADAM_GRAD_F16 1
+
+int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
+                     int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream);
+
+/* Drops the tables cached by fsadam_step and fsadam_grad_pass (synchronises the devices that own them). */
 int fsadam_clear_cache(void);
 
 /* ---- measurement aid: a plain 128-bit copy kernel of known traffic (nbytes read + nbytes

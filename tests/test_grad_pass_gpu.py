@@ -1,0 +1,246 @@
+"""GPU parity of the fused gradient pass (``fsadam_grad_pass`` through the C ABI) against its oracle.
+
+Bars: what is stored (unscaled gradients) and the overflow flag are bit-exact; the max norm is exact
+(a maximum does not round); the sum of squares is within 1e-6 relative of the float64 oracle (the
+device squares in float32, like ``torch.norm(..., dtype=float32)``, and then adds in float64 in a fixed
+order) and bit-identical between runs."""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import _cases as C
+from oracle import grad_oracle as G
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 7, 8, 9, 255, 2047, 2048, 2049, 4095, 4097, 65535, 65536, 65537, 131071, 131072, 131073, 300001]
+
+
+def host_grads(dtype, seed, sizes, scale=1.0):
+    rng = np.random.default_rng(seed)
+    return [(rng.standard_normal(n).astype(np.float32) * np.float32(1e-3 * scale)).astype(dtype) for n in sizes]
+
+
+def run_both(host, device, inv_scale, write_back, misalign=0, scale_on_device=False):
+    from fairscale_amd.grad_pass import grad_pass
+
+    dev = []
+    for h in host:
+        t = torch.from_numpy(h).to(device)
+        if misalign:
+            big = torch.empty(h.size + misalign + 8, dtype=t.dtype, device=device)
+            view = big[misalign:misalign + h.size]
+            view.copy_(t)
+            t = view
+        dev.append(t)
+    inv = torch.tensor([inv_scale], dtype=torch.float32, device=device) if scale_on_device else inv_scale
+    stats = grad_pass(dev, inv, write_back=write_back)
+    torch.cuda.synchronize()
+    want = G.grad_pass_numpy(host, inv_scale, write_back)
+    return dev, stats, want
+
+
+def check(host, dev, stats, want, what):
+    found, ss, mx = want
+    assert stats.found_inf.item() == found, what
+    for i, (h, d) in enumerate(zip(host, dev)):
+        got = d.cpu().numpy()
+        nan = np.isnan(h)
+        assert np.array_equal(np.isnan(got), nan), f"{what} grad[{i}]"
+        assert np.array_equal(got[~nan], h[~nan]), f"{what} grad[{i}] n={h.size}"
+    got_ss, got_mx = stats.sum_squares.item(), stats.abs_max.item()
+    if math.isnan(ss):
+        assert math.isnan(got_ss) and math.isnan(got_mx), what
+    elif math.isinf(ss):
+        assert math.isinf(got_ss) and got_mx == mx, what
+    else:
+        assert abs(got_ss - ss) <= 1e-6 * ss, f"{what}: sum of squares {got_ss!r} vs {ss!r}"
+        assert got_mx == mx, what
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("inv_scale", [1.0, 1.0 / 1024, 1.0 / 3])
+@pytest.mark.parametrize("write_back", [True, False])
+def test_ragged_list_matches_oracle(cuda_device, dtype, inv_scale, write_back):
+    host = host_grads(dtype, 10, SIZES, scale=1.0 / inv_scale)
+    dev, stats, want = run_both(host, cuda_device, inv_scale, write_back)
+    check(host, dev, stats, want, f"{np.dtype(dtype)} inv={inv_scale} wb={write_back}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_misaligned_views_and_device_resident_scale(cuda_device, dtype):
+    host = host_grads(dtype, 11, [5, 4099, 70001, 140001], scale=64.0)
+    dev, stats, want = run_both(host, cuda_device, 1 / 64, True, misalign=1, scale_on_device=True)
+    check(host, dev, stats, want, "misaligned")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_non_finite_at_every_position_of_a_tile(cuda_device, dtype):
+    """One inf or NaN at a time at every lane position of a 16-byte vector, at tile edges and in the
+    ragged tail: flag up, norms inf/NaN, everything else still unscaled."""
+    per_vec = 8 if dtype == np.float16 else 4
+    tile = 64 * per_vec * 4
+    n = 2 * tile + 3 * per_vec + 3
+    positions = list(range(per_vec)) + [tile - 1, tile, tile + per_vec - 1, n - per_vec - 3, n - 2, n - 1]
+    for pos in positions:
+        for bad in (np.inf, np.nan):
+            host = host_grads(dtype, 12, [n, 17], scale=16.0)
+            host[0][pos] = bad
+            dev, stats, want = run_both(host, cuda_device, 1 / 16, True)
+            assert want[0] == 1.0
+            check(host, dev, stats, want, f"{bad} at {pos}")
+    host = host_grads(dtype, 12, [n, 17], scale=16.0)
+    dev, stats, want = run_both(host, cuda_device, 1 / 16, True)
+    assert want[0] == 0.0 and stats.found_inf.item() == 0.0
+
+
+def test_subnormal_half_gradients_are_not_flushed(cuda_device):
+    """Unscaled fp16 gradients below 6.1e-5 are subnormal halves: their squares must still be summed."""
+    host = host_grads(np.float16, 13, [100003, 4099], scale=1e-3)  # ~1e-6: every value subnormal or zero
+    assert all((np.abs(h.astype(np.float32)) < 6.2e-5).all() for h in host) and any((h != 0).any() for h in host)
+    for inv_scale in (1.0, 0.5):
+        dev, stats, want = run_both([h.copy() for h in host], cuda_device, inv_scale, True)
+        assert want[1] > 0
+        assert abs(stats.sum_squares.item() - want[1]) <= 1e-6 * want[1]
+        assert stats.abs_max.item() == want[2] > 0
+
+
+def test_found_inf_is_sticky_and_zero_sized_tensors_are_skipped(cuda_device):
+    from fairscale_amd.grad_pass import grad_pass
+
+    flag = torch.ones(1, device=cuda_device)
+    g = [torch.zeros(0, device=cuda_device), torch.full((1000,), 3.0, device=cuda_device), torch.zeros(0, device=cuda_device)]
+    stats = grad_pass(g, 0.5, found_inf=flag)
+    assert stats.found_inf.item() == 1.0  # never cleared by the pass
+    assert stats.sum_squares.item() == 1000 * 2.25 and stats.abs_max.item() == 1.5
+    assert torch.equal(g[1], torch.full((1000,), 1.5, device=cuda_device))
+    empty = grad_pass([torch.zeros(0, device=cuda_device)], 0.5)
+    assert empty.sum_squares.item() == 0.0 and empty.abs_max.item() == 0.0 and empty.found_inf.item() == 0.0
+
+
+def test_shard_sized_fp16_gradients_against_torch_and_determinism(cuda_device):
+    """1.63e9 fp16 gradients (the shard of the benchmark): norm against torch's float64 sum over
+    chunks, unscale against torch's multiplication, two runs bit-identical."""
+    from fairscale_amd.grad_pass import grad_pass
+
+    n = 1_630_000_000
+    gen = torch.Generator(device=cuda_device).manual_seed(6000)
+    g = torch.empty(n, device=cuda_device, dtype=torch.float16).normal_(0, 1.0, generator=gen)
+    a = grad_pass([g], 1.0 / 1024, write_back=False)
+    b = grad_pass([g], 1.0 / 1024, write_back=False)
+    assert torch.equal(a.sum_squares, b.sum_squares) and torch.equal(a.abs_max, b.abs_max)
+    want_ss, want_mx = 0.0, 0.0
+    for lo in range(0, n, 1 << 27):
+        u = (g[lo:lo + (1 << 27)].float() * (1.0 / 1024)).half().double()
+        want_ss += float((u * u).sum().item())
+        want_mx = max(want_mx, float(u.abs().max().item()))
+        del u
+    assert abs(a.sum_squares.item() - want_ss) <= 1e-6 * want_ss
+    assert a.abs_max.item() == want_mx and a.found_inf.item() == 0.0
+    ref = (g[-5_000_000:].float() * (1.0 / 1024)).half()
+    grad_pass([g], 1.0 / 1024, write_back=True)
+    assert torch.equal(g[-5_000_000:], ref)
+
+
+def test_calc_grad_norm_and_clip_follow_the_reference_contract(cuda_device):
+    """calc_grad_norm / clip_grad_norm_ against the reference's formulas written with torch ops
+    (fairscale/internal/params.py:59-76, fairscale/optim/oss.py:244-302)."""
+    from math import inf
+
+    from fairscale_amd.optim import calc_grad_norm, clip_grad_norm_
+
+    torch.manual_seed(3)
+    for dtype in (torch.float32, torch.float16):
+        params = [torch.nn.Parameter(torch.randn(n, device=cuda_device).to(dtype)) for n in (10, 3001, 200000)]
+        params.append(torch.nn.Parameter(torch.randn(5, device=cuda_device).to(dtype)))  # no gradient: filtered out
+        for p in params[:3]:
+            p.grad = (torch.randn(p.numel(), device=cuda_device) * 0.01).to(dtype)
+        grads = [p.grad for p in params[:3]]
+        want2 = torch.norm(torch.stack([torch.norm(g.detach(), 2.0, dtype=torch.float32) for g in grads]), 2.0).to(dtype)
+        got2 = calc_grad_norm(params, 2.0)
+        assert got2.dtype == dtype and got2.shape == ()
+        assert abs(got2.item() - want2.item()) <= (2e-3 if dtype == torch.float16 else 2e-6) * want2.item()
+        assert calc_grad_norm(params, inf).item() == max(g.abs().max() for g in grads).item()
+        want3 = torch.norm(torch.stack([torch.norm(g.detach(), 3.0, dtype=torch.float32) for g in grads]), 3.0).to(dtype)
+        assert calc_grad_norm(params, 3.0).item() == want3.item()  # other p: torch.norm, as in the reference
+        # clipping: total norm returned, gradients scaled by max_norm / (norm + 1e-6)
+        max_norm = got2.item() / 2
+        before = [g.clone() for g in grads]
+        total = clip_grad_norm_(params, max_norm)
+        assert total.item() == got2.item()
+        coef = torch.tensor(max_norm, dtype=total.dtype, device=total.device) / (total + 1e-6)
+        for g, b in zip(grads, before):
+            assert torch.equal(g, b.clone().mul_(coef))
+        after = calc_grad_norm(params, 2.0).item()
+        assert abs(after - max_norm) <= 5e-3 * max_norm
+        # no clipping needed: untouched
+        snap = [g.clone() for g in grads]
+        clip_grad_norm_(params, 10 * got2.item())
+        assert all(torch.equal(g, s) for g, s in zip(grads, snap))
+    assert calc_grad_norm([torch.nn.Parameter(torch.zeros(3, device=cuda_device))], 2.0).item() == 0.0
+
+
+def test_folding_the_clip_into_the_step_matches_clipping_in_float32(cuda_device):
+    """clip_grad_norm_(fold=True) + Adam.step(scale=...) on fp32 gradients: the step divides by
+    1/clip_coef in registers; clipping first and stepping with scale 1 multiplies by clip_coef and
+    stores. Same mathematics, one rounding apart: parameters agree to 1e-6 relative."""
+    from fairscale_amd.optim import Adam, clip_grad_norm_
+
+    torch.manual_seed(4)
+    base = torch.randn(50000, device=cuda_device) * 0.02
+    grad = torch.randn(50000, device=cuda_device) * 0.1
+    outs = []
+    for fold in (False, True):
+        p = torch.nn.Parameter(base.clone())
+        p.grad = grad.clone()
+        opt = Adam([p], lr=1e-3)
+        if fold:
+            norm, scale = clip_grad_norm_([p], 1.0, fold=True)
+            assert scale > 1.0 and torch.equal(p.grad, grad)
+            opt.step(scale=scale)
+        else:
+            norm = clip_grad_norm_([p], 1.0)
+            opt.step()
+        outs.append((norm.item(), p.detach().clone()))
+    assert outs[0][0] == outs[1][0]
+    assert torch.allclose(outs[0][1], outs[1][1], rtol=1e-6, atol=1e-9)
+
+
+def test_grad_scaler_unscales_through_the_fused_pass(cuda_device):
+    from fairscale_amd.optim import Adam, GradScaler, Precision
+
+    torch.manual_seed(5)
+    w = (torch.randn(64, 32, device=cuda_device) * 0.1).half().requires_grad_()
+    b = torch.zeros(64, device=cuda_device).half().requires_grad_()
+    x = torch.randn(32, device=cuda_device).half()
+    opt = Adam([w, b], lr=1e-2, precision=Precision.MEMORY_EFFICIENT_MIXED_PRECISION)
+    scaler = GradScaler(init_scale=256.0)
+    first = None
+    for i in range(6):
+        opt.zero_grad()
+        loss = (w.mv(x) + b).pow(2).sum()
+        first = loss.item() if first is None else first
+        scaler.scale(loss).backward()
+        scaled = [w.grad.clone(), b.grad.clone()]
+        scaler.unscale_(opt)
+        inv = 1.0 / scaler.get_scale()
+        for g, s in zip((w.grad, b.grad), scaled):
+            assert torch.equal(g, (s.float() * inv).half())
+        norm = scaler.unscaled_grad_norm(opt)
+        want = torch.norm(torch.stack([torch.norm(g.detach(), 2.0, dtype=torch.float32) for g in (w.grad, b.grad)]), 2.0)
+        assert abs(norm.item() - want.item()) <= 2e-6 * want.item()
+        scaler.step(opt)
+        scaler.update()
+    assert loss.item() < first
+    # an overflowing backward: the flag goes up, the step is skipped and the scale backs off
+    opt.zero_grad()
+    w.grad = torch.full_like(w, float("inf"))
+    b.grad = torch.zeros_like(b)
+    before, scale_before = w.detach().clone(), scaler.get_scale()
+    scaler.step(opt)
+    scaler.update()
+    assert torch.equal(w.detach(), before) and scaler.get_scale() == scale_before * 0.5
