@@ -551,6 +551,8 @@ struct Options {
     int64_t groups = 1;         // vectors per lane per stream: 1 or 2
     int64_t lds_throttle = -1;  // bytes of untouched LDS per workgroup (0 = no cap, -1 = per-mode default)
     int64_t xcd_remap = 0;      // 1: contiguous eighth of the tiles per XCD
+    int64_t grad_items = 0;     // gradient pass: 16-byte vectors per lane (2, 4 or 8; 0 = by kind of pass)
+    int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -867,6 +869,8 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
 struct GradPlan {
     int device = -1;
     int dtype = 0;
+    int64_t items = 4;
+    int64_t lds_throttle = 0;
     std::vector<FsGradTensor> rows;
     Layout layout;
     TableSlot slots[kTableSlots];
@@ -878,16 +882,14 @@ struct GradPlan {
     uint64_t lru = 0;
 };
 
-constexpr int kGradItems = 4;        // 16-byte vectors per lane: 4 KiB per wave
-constexpr int kGradThrottle = 13312; // LDS ballast per workgroup for the gradient kernels
 constexpr int kReduceBlocks = 512;
 
 int grad_elem_size(int dtype) { return dtype == FSADAM_GRAD_F16 ? 2 : 4; }
-int64_t grad_tile_elems(int dtype) { return 64 * (16 / grad_elem_size(dtype)) * kGradItems; }
+int64_t grad_tile_elems(int dtype, int64_t items) { return 64 * (16 / grad_elem_size(dtype)) * items; }
 
-Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype) {
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items) {
     Layout L;
-    L.tile_elems = grad_tile_elems(dtype);
+    L.tile_elems = grad_tile_elems(dtype, items);
     int64_t min_large = 0;
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = grads[t].numel;
@@ -922,8 +924,16 @@ void grad_plan_free(GradPlan* plan) {
     delete plan;
 }
 
+// Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
+// a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
+void grad_shape(bool writes, int64_t* items, int64_t* lds) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
+    *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 13312 : 16384);
+}
+
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
-    const Layout L = grad_layout(grads, n, plan->dtype);
+    const Layout L = grad_layout(grads, n, plan->dtype, plan->items);
     const int64_t k = L.large_chunk_elems / L.tile_elems;
     const int64_t n_blocks = L.n_large_descs * k + L.n_small_descs;
     if (L.n_large_descs * k > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
@@ -999,12 +1009,20 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     GradPartial* first = plan->d_partials;
     GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
     GradPartial* total = second + kReduceBlocks;
-    if (large_blocks > 0)
-        hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, kGradItems>), dim3((uint32_t)large_blocks), dim3(64), kGradThrottle, stream,
-                           slot.d_table, (uint32_t)log2k, inv_scale, inv_scale_dev, write_back, first);
-    if (L.n_small_descs > 0)
-        hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, kGradItems>), dim3((uint32_t)L.n_small_descs), dim3(64), kGradThrottle, stream,
-                           slot.d_table + L.n_large_descs, 0u, inv_scale, inv_scale_dev, write_back, first + large_blocks);
+#define FS_GRAD_LAUNCH(ITEMS)                                                                                                   \
+    do {                                                                                                                        \
+        if (large_blocks > 0)                                                                                                   \
+            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)large_blocks), dim3(64), lds, stream,          \
+                               slot.d_table, (uint32_t)log2k, inv_scale, inv_scale_dev, write_back, first);                    \
+        if (L.n_small_descs > 0)                                                                                                \
+            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)L.n_small_descs), dim3(64), lds, stream,       \
+                               slot.d_table + L.n_large_descs, 0u, inv_scale, inv_scale_dev, write_back, first + large_blocks); \
+    } while (0)
+    const size_t lds = (size_t)plan->lds_throttle;
+    if (plan->items == 2) FS_GRAD_LAUNCH(2);
+    else if (plan->items == 8) FS_GRAD_LAUNCH(8);
+    else FS_GRAD_LAUNCH(4);
+#undef FS_GRAD_LAUNCH
     FS_HIP(hipGetLastError());
     // two fixed-shape reduction steps, then publish (also when the list holds no element: everything is zero)
     const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_blocks, 1024)));
@@ -1020,7 +1038,7 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
 }
 
 std::vector<GradPlan*> g_grad_cache;
-constexpr size_t kGradCacheWays = 4;
+constexpr size_t kGradCacheWays = 6;
 
 bool same_grad_rows(const GradPlan* plan, const FsGradTensor* grads, int64_t n) {
     if ((int64_t)plan->rows.size() != n) return false;
@@ -1083,6 +1101,12 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "xcd_remap") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "xcd_remap must be 0 or 1");
         g_opt.xcd_remap = value;
+    } else if (k == "grad_items") {
+        if (value != 0 && value != 2 && value != 4 && value != 8) return fail(FSADAM_EINVAL, "grad_items must be 0 (automatic), 2, 4 or 8");
+        g_opt.grad_items = value;
+    } else if (k == "grad_lds_throttle") {
+        if (value < -1 || value > 65536) return fail(FSADAM_EINVAL, "grad_lds_throttle must be -1 (automatic) or in [0, 65536] bytes");
+        g_opt.grad_lds_throttle = value;
     } else {
         return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
     }
@@ -1097,6 +1121,8 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "groups") *value = g_opt.groups;
     else if (k == "lds_throttle") *value = g_opt.lds_throttle;
     else if (k == "xcd_remap") *value = g_opt.xcd_remap;
+    else if (k == "grad_items") *value = g_opt.grad_items;
+    else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
     return FSADAM_OK;
 }
@@ -1241,11 +1267,14 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    int64_t cur_items, cur_lds;
+    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
-        if (c->device == dev && c->dtype == grad_dtype && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+        if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
+            same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -1254,6 +1283,8 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
             if (!fresh) return fail(FSADAM_ENOMEM, "out of host memory");
             fresh->device = dev;
             fresh->dtype = grad_dtype;
+            fresh->items = cur_items;
+            fresh->lds_throttle = cur_lds;
             if (g_grad_cache.size() >= kGradCacheWays) {
                 size_t oldest = 0;
                 for (size_t i = 1; i < g_grad_cache.size(); ++i) if (g_grad_cache[i]->lru < g_grad_cache[oldest]->lru) oldest = i;
@@ -1264,6 +1295,8 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
             }
             victim = fresh;
         }
+        victim->items = cur_items;
+        victim->lds_throttle = cur_lds;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;

@@ -108,6 +108,9 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
  *                   per-mode default (13-16 KiB, default)
  *   "xcd_remap"     0/1: hand each XCD a contiguous eighth of the tiles (default 0)
+ *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
+ *                   4 for one that writes the gradients back (default 0)
+ *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
  * Affects plans whose tensors are set after the call. */
 int fsadam_set_option(const char* name, int64_t value);
 int fsadam_get_option(const char* name, int64_t* value);
