@@ -15,6 +15,7 @@ FULL_PRECISION = 0
 MIXED_PRECISION = 1
 MEMORY_EFFICIENT_MIXED_PRECISION = 2
 PURE_FP16 = 3
+FULL_PRECISION_FP16_COPY = 4
 
 ABI_VERSION = 1
 

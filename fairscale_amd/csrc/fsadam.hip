@@ -109,7 +109,15 @@ struct ModeTraits<FSADAM_PURE_FP16> {
     static constexpr int kElems = 8;
 };
 
+template <>
+struct ModeTraits<FSADAM_FULL_PRECISION_FP16_COPY> {
+    using P = float; using G = float; using S = float;
+    static constexpr bool kCopy = true, kScaled = false;
+    static constexpr int kElems = 4;
+};
+
 constexpr int mode_elems(int mode) { return mode == FSADAM_PURE_FP16 ? 8 : 4; }
+constexpr bool mode_has_copy(int mode) { return mode == FSADAM_MIXED_PRECISION || mode == FSADAM_FULL_PRECISION_FP16_COPY; }
 
 // --------------------------------------------------------------------------------------------
 // device code
@@ -561,6 +569,7 @@ struct Options {
 int64_t default_lds_throttle(int mode) {
     switch (mode) {
         case FSADAM_FULL_PRECISION: return 16384;
+        case FSADAM_FULL_PRECISION_FP16_COPY: return 16384;
         case FSADAM_MIXED_PRECISION: return 15360;
         case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
         default: return 13312;
@@ -570,11 +579,11 @@ Options g_opt;
 std::mutex g_mutex;        // guards g_opt
 std::mutex g_cache_mutex;  // guards the fsadam_step table cache
 
-bool valid_mode(int mode) { return mode >= FSADAM_FULL_PRECISION && mode <= FSADAM_PURE_FP16; }
+bool valid_mode(int mode) { return mode >= FSADAM_FULL_PRECISION && mode <= FSADAM_FULL_PRECISION_FP16_COPY; }
 
-int size_p(int mode) { return (mode == FSADAM_FULL_PRECISION || mode == FSADAM_MIXED_PRECISION) ? 4 : 2; }
+int size_p(int mode) { return (mode == FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION || mode == FSADAM_PURE_FP16) ? 2 : 4; }
 int size_s(int mode) { return mode == FSADAM_PURE_FP16 ? 2 : 4; }
-int size_g(int mode) { return mode == FSADAM_FULL_PRECISION ? 4 : 2; }
+int size_g(int mode) { return (mode == FSADAM_FULL_PRECISION || mode == FSADAM_FULL_PRECISION_FP16_COPY) ? 4 : 2; }
 
 bool aligned_to(const void* ptr, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(ptr) & (bytes - 1)) == 0; }
 
@@ -598,11 +607,11 @@ int validate_rows(const FsAdamTensor* tensors, int64_t n, int mode) {
         if (r.numel < 0) return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": negative numel");
         if (r.numel == 0) continue;
         if (!r.p || !r.m || !r.v || !r.g) return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": NULL p/m/v/g pointer");
-        if (mode == FSADAM_MIXED_PRECISION && !r.p_copy)
-            return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": MIXED_PRECISION needs p_copy");
+        if (mode_has_copy(mode) && !r.p_copy)
+            return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": this mode needs p_copy");
         // anything less than element alignment cannot be a tensor of that dtype
         if (!aligned_to(r.p, size_p(mode)) || !aligned_to(r.m, size_s(mode)) || !aligned_to(r.v, size_s(mode)) ||
-            !aligned_to(r.g, size_g(mode)) || (mode == FSADAM_MIXED_PRECISION && !aligned_to(r.p_copy, 2)))
+            !aligned_to(r.g, size_g(mode)) || (mode_has_copy(mode) && !aligned_to(r.p_copy, 2)))
             return fail(FSADAM_EINVAL, "tensor " + std::to_string(t) + ": pointer not aligned to its element size");
     }
     return FSADAM_OK;
@@ -612,7 +621,7 @@ int validate_rows(const FsAdamTensor* tensors, int64_t n, int mode) {
 bool row_vector_ok(const FsAdamTensor& r, int mode) {
     const uintptr_t e = mode_elems(mode);
     return aligned_to(r.p, e * size_p(mode)) && aligned_to(r.m, e * size_s(mode)) && aligned_to(r.v, e * size_s(mode)) &&
-           aligned_to(r.g, e * size_g(mode)) && (mode != FSADAM_MIXED_PRECISION || aligned_to(r.p_copy, e * 2));
+           aligned_to(r.g, e * size_g(mode)) && (!mode_has_copy(mode) || aligned_to(r.p_copy, e * 2));
 }
 
 int64_t floor_pow2(int64_t x) {
@@ -720,7 +729,7 @@ void fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t chunk_e
         d.m = advance(r.m, first, size_s(mode));
         d.v = advance(r.v, first, size_s(mode));
         d.g = advance(r.g, first, size_g(mode));
-        d.p_copy = (mode == FSADAM_MIXED_PRECISION) ? advance(r.p_copy, first, 2) : nullptr;
+        d.p_copy = mode_has_copy(mode) ? advance(r.p_copy, first, 2) : nullptr;
         d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - first);
         d.vector_ok = vec ? 1u : 0u;
         d.pad = 0;
@@ -761,6 +770,8 @@ int launch_mode(int mode, const ChunkDesc* table, int64_t n_descs, int log2k, co
         case FSADAM_MIXED_PRECISION: return launch_shape<FSADAM_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
         case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION:
             return launch_shape<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
+        case FSADAM_FULL_PRECISION_FP16_COPY:
+            return launch_shape<FSADAM_FULL_PRECISION_FP16_COPY>(table, n_descs, log2k, opt, s, found_inf, stream);
         default: return launch_shape<FSADAM_PURE_FP16>(table, n_descs, log2k, opt, s, found_inf, stream);
     }
 }

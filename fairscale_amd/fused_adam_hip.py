@@ -32,9 +32,10 @@ def mode_of_lists(tensor_lists: Sequence[Sequence[torch.Tensor]]) -> int:
     if m != v:
         raise RuntimeError("exp_avg and exp_avg_sq must have the same dtype")  # kernel.cu:167
     if depth == 5:
-        if p != torch.float32 or g != torch.float16 or tensor_lists[4][0].dtype != torch.float16 or m != torch.float32:
-            raise RuntimeError("mixed precision expects fp32 params/state with fp16 grads and fp16 output params")  # kernel.cu:174-176
-        return _cabi.MIXED_PRECISION
+        if p != torch.float32 or tensor_lists[4][0].dtype != torch.float16 or m != torch.float32 or g not in (torch.float16, torch.float32):
+            raise RuntimeError("five lists expect fp32 params/state, fp16 or fp32 grads and fp16 output params")  # kernel.cu:174-176
+        # fp32 grads with a copy-out have no case in the reference (its asserts require fp16 grads): extension
+        return _cabi.MIXED_PRECISION if g == torch.float16 else _cabi.FULL_PRECISION_FP16_COPY
     if p != g:
         raise RuntimeError("params and grads must have the same dtype")  # kernel.cu:196
     if p == torch.float32:
@@ -55,6 +56,7 @@ _MODE_DTYPES = {
     _cabi.MIXED_PRECISION: (torch.float32, torch.float32, torch.float32, torch.float16, torch.float16),
     _cabi.MEMORY_EFFICIENT_MIXED_PRECISION: (torch.float16, torch.float32, torch.float32, torch.float16),
     _cabi.PURE_FP16: (torch.float16, torch.float16, torch.float16, torch.float16),
+    _cabi.FULL_PRECISION_FP16_COPY: (torch.float32, torch.float32, torch.float32, torch.float32, torch.float16),
 }
 
 

@@ -191,16 +191,34 @@ class Adam(torch.optim.Optimizer):
             self._flags[device] = flag
         return flag
 
+    def attach_fp16_copies(self, copies: Optional[Dict[torch.Tensor, torch.Tensor]]) -> None:
+        """FULL_PRECISION only.  ``copies`` maps parameters to fp16 tensors of the same shape that the
+        step then overwrites with ``half(p)`` in the same pass (None detaches).  This is the cast FSDP
+        redoes before every forward (``_cast_fp32_param_shards_to_fp16``,
+        ``fully_sharded_data_parallel.py:2253-2267``); fused, it costs 2 written bytes per parameter
+        instead of a separate 4-byte read and 2-byte write.  Every parameter that gets a gradient must
+        have a copy attached."""
+        if copies is not None:
+            if self.precision is not Precision.FULL_PRECISION:
+                raise RuntimeError("fp16 copies can only be attached in FULL_PRECISION (MIXED_PRECISION already writes them)")
+            for p, c in copies.items():
+                if c.dtype != torch.float16 or c.numel() != p.numel() or c.device != p.device or not c.is_contiguous():
+                    raise RuntimeError("an fp16 copy must be a contiguous float16 tensor with the parameter's numel and device")
+        self._fp16_copies = dict(copies) if copies is not None else None
+        self._plans_invalidate()
+
     def _gather(self, gi: int, group: Dict[str, Any]):
         """The per-parameter walk of adam.py:207-254: lazy state, step counters, tensor lists per device.
         Also (re)builds the group's fast-path cache when every parameter took part and shares one device."""
         mixed = self.mixed_precision
+        copies = self.__dict__.get("_fp16_copies")
         state_map, optim_type = self.state, self.optim_type
         masters = self.fp32_param_groups[gi]["params"] if mixed else None
         batches: Dict[torch.device, List[List[torch.Tensor]]] = {}
         states: List[dict] = []
         step_no = None
         params = group["params"]
+        depth = 5 if (mixed or copies is not None) else 4
         for pj, p in enumerate(params):
             grad = p.grad
             if grad is None:
@@ -216,17 +234,22 @@ class Adam(torch.optim.Optimizer):
             states.append(state)
             lists = batches.get(p.device)
             if lists is None:
-                lists = batches[p.device] = [[] for _ in range(5 if mixed else 4)]
+                lists = batches[p.device] = [[] for _ in range(depth)]
             lists[0].append(masters[pj] if mixed else p)
             lists[1].append(state["exp_avg"])
             lists[2].append(state["exp_avg_sq"])
             lists[3].append(grad)
             if mixed:
                 lists[4].append(p)
+            elif copies is not None:
+                if p not in copies:
+                    raise RuntimeError("a parameter with a gradient has no fp16 copy attached")
+                lists[4].append(copies[p])
         caches = self.__dict__.setdefault("_group_cache", {})
         if len(states) == len(params) and len(batches) == 1:
-            device = next(iter(batches))
-            caches[gi] = (params, len(params), states, masters, device)
+            device, lists = next(iter(batches.items()))
+            outs = lists[4] if depth == 5 else None
+            caches[gi] = (params, len(params), states, masters, outs, device)
         else:
             caches.pop(gi, None)
         return batches, step_no
@@ -238,7 +261,7 @@ class Adam(torch.optim.Optimizer):
         cache = self.__dict__.get("_group_cache", {}).get(gi)
         if cache is None:
             return None, None
-        params, count, states, masters, device = cache
+        params, count, states, masters, outs, device = cache
         if group["params"] is not params or len(params) != count or count == 0:
             return None, None
         if self.state.get(params[-1]) is not states[-1] or self.state.get(params[0]) is not states[0]:
@@ -257,8 +280,8 @@ class Adam(torch.optim.Optimizer):
         for st in states:
             st["step"] += 1
         lists = [masters if masters is not None else params, m_list, v_list, grads]
-        if masters is not None:
-            lists.append(params)
+        if outs is not None:
+            lists.append(outs)
         return {device: lists}, states[-1]["step"]
 
     def step(self, closure: Optional[Callable[[], float]] = None, *, scale: float = 1.0) -> Optional[float]:
@@ -272,6 +295,8 @@ class Adam(torch.optim.Optimizer):
         self.__dict__.setdefault("_plans", {})  # absent after unpickling
         self.__dict__.setdefault("_flags", {})
         native_mode = _NATIVE_MODE[self.precision]
+        if self.__dict__.get("_fp16_copies") is not None:
+            native_mode = _cabi.FULL_PRECISION_FP16_COPY
         watch_overflow = self.precision is Precision.PURE_FP16
 
         for gi, group in enumerate(self.param_groups):

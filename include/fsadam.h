@@ -31,6 +31,11 @@ extern "C" {
 #define FSADAM_MIXED_PRECISION 1                        /* f32    f16    f32    f16 (written)     */
 #define FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION 2       /* f16    f16    f32    -                 */
 #define FSADAM_PURE_FP16 3                              /* f16    f16    f16    -   (state*scale) */
+/* Not a combination the reference dispatches on: the fp32 step of an FSDP shard with the fp16 copy of
+ * the parameters written in the same pass -- what FullyShardedDataParallel._cast_fp32_param_shards_to_fp16
+ * (fairscale/nn/data_parallel/fully_sharded_data_parallel.py:2253-2267) recomputes before the next
+ * forward: p_copy = half(p), one rounding of the stored fp32 value (kernel.cu:114,129).              */
+#define FSADAM_FULL_PRECISION_FP16_COPY 4               /* f32    f32    f32    f16 (written)     */
 
 /* eps placement (adamMode_t, fused_adam_cuda_kernel.cu:16-19) */
 #define FSADAM_EPS_INSIDE_SQRT 0
@@ -45,13 +50,14 @@ extern "C" {
 /* One row of the tensor list: replaces column t of the reference's tensor_lists[d][t]
  * (TensorListMetadata, fairscale/clib/fused_adam_cuda/multi_tensor_apply.cuh:18-25).  numel is
  * 64-bit (the reference truncates to int, multi_tensor_apply.cuh:21,80).  Every pointer must address
- * numel contiguous elements of the dtype the mode implies.  p_copy is read only in MIXED mode. */
+ * numel contiguous elements of the dtype the mode implies.  p_copy is used only by the two modes that
+ * write an fp16 copy (MIXED_PRECISION, FULL_PRECISION_FP16_COPY). */
 typedef struct FsAdamTensor {
     void* p;        /* parameters (fp32 master copy in MIXED)                       */
     void* m;        /* exp_avg                                                      */
     void* v;        /* exp_avg_sq                                                   */
     const void* g;  /* gradients                                                    */
-    void* p_copy;   /* MIXED: fp16 parameters to overwrite; otherwise ignored/NULL  */
+    void* p_copy;   /* copy-out modes: fp16 parameters to overwrite; else ignored    */
     int64_t numel;
 } FsAdamTensor;
 

@@ -46,7 +46,10 @@ enum {
     ORACLE_FULL_PRECISION = 0,                   /* p f32, g f32, m/v f32            kernel.cu:197-216 */
     ORACLE_MIXED_PRECISION = 1,                  /* p f32, g f16, m/v f32, p_copy f16 kernel.cu:172-193 */
     ORACLE_MEMORY_EFFICIENT_MIXED_PRECISION = 2, /* p f16, g f16, m/v f32            kernel.cu:217-237 */
-    ORACLE_PURE_FP16 = 3                         /* p f16, g f16, m/v f16            kernel.cu:238-256 */
+    ORACLE_PURE_FP16 = 3,                        /* p f16, g f16, m/v f16            kernel.cu:238-256 */
+    /* extension, no dispatch case in the reference: the fp32 step with the DEPTH==5 copy-out of
+     * kernel.cu:114,129 (p_copy = half(stored p)) applied to fp32 gradients */
+    ORACLE_FULL_PRECISION_FP16_COPY = 4
 };
 
 /* ---- IEEE binary16 <-> binary32, software, independent of the host's F16C support ---- */
@@ -155,9 +158,10 @@ int fsadam_oracle_step(int mode, void* p, void* m, void* v, const void* g, void*
         case ORACLE_MIXED_PRECISION: p_half = 0; g_half = 1; s_half = 0; break;
         case ORACLE_MEMORY_EFFICIENT_MIXED_PRECISION: p_half = 1; g_half = 1; s_half = 0; break;
         case ORACLE_PURE_FP16: p_half = 1; g_half = 1; s_half = 1; break;
+        case ORACLE_FULL_PRECISION_FP16_COPY: p_half = 0; g_half = 0; s_half = 0; break;
         default: return -1;
     }
-    const int depth5 = (mode == ORACLE_MIXED_PRECISION);
+    const int depth5 = (mode == ORACLE_MIXED_PRECISION || mode == ORACLE_FULL_PRECISION_FP16_COPY);
     if (depth5 && p_copy == 0) return -1;
     const float step_size = fsadam_oracle_step_size(lr, b1, b2, step, bias_correction);
     const float one_minus_b1 = 1 - b1; /* float subtraction, kernel.cu:97,118 */

@@ -25,12 +25,14 @@ FULL_PRECISION = 0
 MIXED_PRECISION = 1
 MEMORY_EFFICIENT_MIXED_PRECISION = 2
 PURE_FP16 = 3
+FULL_PRECISION_FP16_COPY = 4  # extension: fp32 step + fp16 copy of p (see adam_oracle.c)
 
 MODE_NAMES = {
     FULL_PRECISION: "FULL_PRECISION",
     MIXED_PRECISION: "MIXED_PRECISION",
     MEMORY_EFFICIENT_MIXED_PRECISION: "MEMORY_EFFICIENT_MIXED_PRECISION",
     PURE_FP16: "PURE_FP16",
+    FULL_PRECISION_FP16_COPY: "FULL_PRECISION_FP16_COPY",
 }
 
 # (param dtype, grad dtype, state dtype) per mode: fused_adam_cuda_kernel.cu:172-256
@@ -39,10 +41,12 @@ MODE_DTYPES = {
     MIXED_PRECISION: (np.float32, np.float16, np.float32),
     MEMORY_EFFICIENT_MIXED_PRECISION: (np.float16, np.float16, np.float32),
     PURE_FP16: (np.float16, np.float16, np.float16),
+    FULL_PRECISION_FP16_COPY: (np.float32, np.float32, np.float32),
 }
 
 # algorithmic bytes per element: reads p,m,v,g + writes p,m,v(,p_copy)
-MODE_BYTES = {FULL_PRECISION: 28, MIXED_PRECISION: 28, MEMORY_EFFICIENT_MIXED_PRECISION: 22, PURE_FP16: 14}
+MODE_BYTES = {FULL_PRECISION: 28, MIXED_PRECISION: 28, MEMORY_EFFICIENT_MIXED_PRECISION: 22, PURE_FP16: 14,
+              FULL_PRECISION_FP16_COPY: 30}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "_build", "libadam_oracle.so")
@@ -125,7 +129,7 @@ def step_c(mode: int, p: np.ndarray, m: np.ndarray, v: np.ndarray, g: np.ndarray
     n = p.size
     assert m.size == n and v.size == n and g.size == n
     pc = None
-    if mode == MIXED_PRECISION:
+    if mode in (MIXED_PRECISION, FULL_PRECISION_FP16_COPY):
         assert p_copy is not None
         _check(p_copy, np.float16, "p_copy")
         assert p_copy.size == n
@@ -184,7 +188,7 @@ def step_numpy(mode: int, p: np.ndarray, m: np.ndarray, v: np.ndarray, g: np.nda
         new_p = in_p - ss * update
         assert new_p.dtype == f
         p[...] = new_p.astype(p.dtype)
-        if mode == MIXED_PRECISION:
+        if mode in (MIXED_PRECISION, FULL_PRECISION_FP16_COPY):
             p_copy[...] = p.astype(np.float16)  # from the stored fp32 p: kernel.cu:129
 
 

@@ -310,6 +310,37 @@ def test_scale_keyword_divides_the_gradients(oracle, api, cuda_device):
         assert torch.equal(a, b)
 
 
+def test_attached_fp16_copies_follow_the_fp32_parameters(api, cuda_device):
+    """attach_fp16_copies: the step leaves half(p) in the attached tensors, parameters and state are those
+    of a plain FULL_PRECISION optimizer bit for bit; detaching stops the writes."""
+    Adam, _, Precision = api
+    torch.manual_seed(7)
+    base = [torch.randn(n, device=cuda_device) * 0.02 for n in (10, 3000, 150000)]
+    grads = [[torch.randn_like(b) * 1e-3 for b in base] for _ in range(3)]
+    plain = [b.clone().requires_grad_() for b in base]
+    fused = [b.clone().requires_grad_() for b in base]
+    copies = {p: torch.zeros(p.numel(), dtype=torch.float16, device=cuda_device) for p in fused}
+    opt_a, opt_b = Adam(plain, weight_decay=0.01), Adam(fused, weight_decay=0.01)
+    opt_b.attach_fp16_copies(copies)
+    for step_grads in grads:
+        for p, q, g in zip(plain, fused, step_grads):
+            p.grad, q.grad = g.clone(), g.clone()
+        opt_a.step()
+        opt_b.step()
+        for p, q in zip(plain, fused):
+            assert torch.equal(p, q) and torch.equal(copies[q], q.detach().half())
+            assert torch.equal(opt_a.state[p]["exp_avg_sq"], opt_b.state[q]["exp_avg_sq"])
+    opt_b.attach_fp16_copies(None)
+    snapshot = {q: copies[q].clone() for q in fused}
+    opt_b.step()
+    assert all(torch.equal(copies[q], snapshot[q]) for q in fused)
+    w16 = torch.zeros(4, device=cuda_device).half().requires_grad_()
+    with pytest.raises(RuntimeError, match="FULL_PRECISION"):
+        Adam([w16], precision=Precision.PURE_FP16).attach_fp16_copies({w16: torch.zeros(4, dtype=torch.float16, device=cuda_device)})
+    with pytest.raises(RuntimeError, match="float16"):
+        opt_b.attach_fp16_copies({fused[0]: torch.zeros(10, device=cuda_device)})
+
+
 def test_table_is_sent_again_only_when_a_pointer_moves(api, cuda_device):
     Adam, _, _ = api
     params = [torch.randn(n, device=cuda_device).requires_grad_() for n in (10, 3000, 200000)]

@@ -56,7 +56,8 @@ def test_abi_version_and_constants():
     for name, a, b in [("FSADAM_FULL_PRECISION", _cabi.FULL_PRECISION, O.FULL_PRECISION),
                        ("FSADAM_MIXED_PRECISION", _cabi.MIXED_PRECISION, O.MIXED_PRECISION),
                        ("FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION", _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, O.MEMORY_EFFICIENT_MIXED_PRECISION),
-                       ("FSADAM_PURE_FP16", _cabi.PURE_FP16, O.PURE_FP16)]:
+                       ("FSADAM_PURE_FP16", _cabi.PURE_FP16, O.PURE_FP16),
+                       ("FSADAM_FULL_PRECISION_FP16_COPY", _cabi.FULL_PRECISION_FP16_COPY, O.FULL_PRECISION_FP16_COPY)]:
         assert header_define(name) == a == b
     assert header_define("FSADAM_EPS_INSIDE_SQRT") == 0 and header_define("FSADAM_EPS_OUTSIDE_SQRT") == 1
     assert ctypes.sizeof(_cabi.FsAdamTensor) == 48  # five pointers and an int64, no padding
@@ -156,6 +157,7 @@ def test_bad_arguments_return_einval_before_touching_a_device():
     cases = [
         (rows(good), 0, _cabi.FULL_PRECISION, "empty"),               # multi_tensor_apply.cuh:51
         (rows(good), 1, 7, "unknown precision mode"),
+        (rows(good), 1, _cabi.FULL_PRECISION_FP16_COPY, "needs p_copy"),
         (None, 1, _cabi.FULL_PRECISION, "NULL"),
         (rows((A, A, A, A, 0, -5)), 1, _cabi.FULL_PRECISION, "negative numel"),
         (rows((0, A, A, A, 0, 16)), 1, _cabi.FULL_PRECISION, "NULL p/m/v/g"),
@@ -209,8 +211,9 @@ def test_mode_dispatch_follows_the_reference():
     assert fused_adam_hip.mode_of_lists(_lists(f32, f16, f32, copy=True)) == _cabi.MIXED_PRECISION
     assert fused_adam_hip.mode_of_lists(_lists(f16, f16, f32)) == _cabi.MEMORY_EFFICIENT_MIXED_PRECISION
     assert fused_adam_hip.mode_of_lists(_lists(f16, f16, f16)) == _cabi.PURE_FP16
+    assert fused_adam_hip.mode_of_lists(_lists(f32, f32, f32, copy=True)) == _cabi.FULL_PRECISION_FP16_COPY  # extension
     for bad in (_lists(f32, f16, f32), _lists(f32, f32, f16), _lists(torch.bfloat16, torch.bfloat16, f32),
-                _lists(f16, f16, torch.float64), _lists(f32, f32, f32, copy=True), _lists(f32, f32, f32)[:3], [[], [], [], []]):
+                _lists(f16, f16, torch.float64), _lists(f16, f16, f32, copy=True), _lists(f32, f32, f32)[:3], [[], [], [], []]):
         with pytest.raises(RuntimeError):
             fused_adam_hip.mode_of_lists(bad)
 

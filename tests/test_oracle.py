@@ -255,6 +255,25 @@ def test_mixed_equals_full_on_widened_grads_and_copy_is_half_of_master(oracle):
     assert np.array_equal(pc, pm.astype(np.float16))  # one rounding of the stored fp32 value (kernel.cu:129)
 
 
+def test_fp16_copy_extension_is_the_full_step_plus_one_rounding(oracle):
+    """Mode 4 (fp32 step with the fp16 copy-out of kernel.cu:114,129 applied to fp32 gradients): p, m, v are
+    those of FULL_PRECISION bit for bit and the copy is numpy's half(p)."""
+    rng = np.random.default_rng(24)
+    p0 = (rng.standard_normal(5000) * 0.02).astype(np.float32)
+    gs = [(rng.standard_normal(5000) * 1e-3).astype(np.float32) for _ in range(3)]
+    pf, mf, vf, _, _ = _run(oracle, FULL, p0, gs, decay=0.01, **HY)
+    p, m, v = p0.copy(), np.zeros(5000, np.float32), np.zeros(5000, np.float32)
+    c = np.zeros(5000, np.float16)
+    for t_, g in enumerate(gs, start=1):
+        oracle.step_c(oracle.FULL_PRECISION_FP16_COPY, p, m, v, g, c, step=t_, decay=0.01, **HY)
+        assert np.array_equal(c, p.astype(np.float16))
+    assert np.array_equal(p, pf) and np.array_equal(m, mf) and np.array_equal(v, vf)
+    p2, m2, v2, c2 = p0.copy(), np.zeros(5000, np.float32), np.zeros(5000, np.float32), np.zeros(5000, np.float16)
+    for t_, g in enumerate(gs, start=1):
+        oracle.step_numpy(oracle.FULL_PRECISION_FP16_COPY, p2, m2, v2, g, c2, step=t_, decay=0.01, **HY)
+    assert np.array_equal(p2, p) and np.array_equal(c2, c)
+
+
 def test_memory_efficient_is_full_with_one_rounding_of_p(oracle):
     """One step from the same inputs: fp16 p out == half(fp32 result of the FULL step on widened inputs)."""
     rng = np.random.default_rng(23)

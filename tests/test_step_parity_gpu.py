@@ -173,6 +173,33 @@ def test_c2_gpt2_small_mixed_precision(oracle, cuda_device):
         assert torch.equal(p32.half(), p16)
 
 
+def test_full_precision_with_fp16_copy_out(oracle, cuda_device):
+    """The extension mode for FSDP-style shards: fp32 p, g, m, v plus an fp16 copy of p written in the
+    same pass.  p, m, v and the copy against the oracle, ragged sizes, one misaligned copy buffer."""
+    from fairscale_amd import fused_adam_hip
+
+    sizes = [1, 5, 255, 257, 4099, 70001, 131072, 200003]
+    host = C.Tensors(FULL, sizes, 4800)
+    copies = [np.zeros(n, np.float16) for n in sizes]
+    dev = GpuList(host, cuda_device)
+    dcopies = [torch.zeros(n, dtype=torch.float16, device=cuda_device) for n in sizes]
+    big = torch.zeros(sizes[5] + 16, dtype=torch.float16, device=cuda_device)
+    dcopies[5] = big[3:3 + sizes[5]]  # 6 bytes into its allocation: that tensor takes the element-wise path
+    flag = torch.zeros(1, device=cuda_device)
+    for step in range(1, 4):
+        grads = host.grads(step)
+        kw = dict(DEFAULT, decay=0.01, step=step)
+        g = to_gpu(grads, cuda_device)
+        fused_adam_hip.adam(65536, None, [dev.p, dev.m, dev.v, g, dcopies], kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], 1.0, 1.0,
+                            flag, step, 1, 1, 0.01)
+        torch.cuda.synchronize()
+        for i in range(len(sizes)):
+            oracle.step_c(oracle.FULL_PRECISION_FP16_COPY, host.p[i], host.m[i], host.v[i], grads[i], copies[i], **kw)
+        compare(host, dev, f"fp16-copy step {step}")
+        for i, (want, got) in enumerate(zip(copies, dcopies)):
+            assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), f"copy[{i}] step {step}"
+
+
 def test_nonfinite_grads_propagate_without_flag(oracle, cuda_device):
     """inf / NaN gradients flow into p, m, v in the fp32-state modes and never raise the flag
     (only the fp16-state branch writes it, fused_adam_cuda_kernel.cu:103-105)."""
