@@ -278,9 +278,11 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
 
     uint32_t block = blockIdx.x;
     if (xcd_stride) {
-        // Consecutive workgroups go to consecutive XCDs (eight L2s).  Give XCD x the x-th contiguous
-        // eighth of the tiles instead of every eighth tile.
-        block = (block & 7u) * xcd_stride + (block >> 3);
+        // Consecutive workgroups go to consecutive XCDs (eight L2s).  Regroup so that XCD x gets runs of
+        // `xcd_stride` consecutive tiles: within a group of 8*run workgroups, workgroup b takes tile
+        // (b % 8) * run + (b / 8) % run.
+        const uint32_t group = block / (8u * xcd_stride), in_group = block % (8u * xcd_stride);
+        block = group * 8u * xcd_stride + (in_group & 7u) * xcd_stride + (in_group >> 3);
         if (block >= n_blocks) return;
     }
     const uint32_t chunk = block >> log2k;
@@ -558,7 +560,7 @@ struct Options {
     int64_t block = 64;         // threads per workgroup: 64, 128 or 256
     int64_t groups = 1;         // vectors per lane per stream: 1 or 2
     int64_t lds_throttle = -1;  // bytes of untouched LDS per workgroup (0 = no cap, -1 = per-mode default)
-    int64_t xcd_remap = 0;      // 1: contiguous eighth of the tiles per XCD
+    int64_t xcd_remap = 0;      // 0: tiles in dispatch order; R > 0: each XCD takes runs of R consecutive tiles
     int64_t grad_items = 0;     // gradient pass: 16-byte vectors per lane (2, 4 or 8; 0 = by kind of pass)
     int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
 };
@@ -743,9 +745,9 @@ int launch_tiles(const ChunkDesc* table, int64_t n_descs, int log2k, const Optio
     const int64_t n_blocks = n_descs << log2k;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
     uint32_t grid = (uint32_t)n_blocks, xcd_stride = 0;
-    if (opt.xcd_remap) {
-        xcd_stride = (uint32_t)ceil_div(n_blocks, 8);
-        grid = xcd_stride * 8;
+    if (opt.xcd_remap) {  // value = tiles per run; 1 would be the identity
+        xcd_stride = (uint32_t)std::min<int64_t>(opt.xcd_remap, ceil_div(n_blocks, 8));
+        grid = (uint32_t)(ceil_div(n_blocks, 8 * (int64_t)xcd_stride) * 8 * xcd_stride);
     }
     hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table,
                        (uint32_t)log2k, (uint32_t)n_blocks, xcd_stride, s, found_inf);
@@ -1110,7 +1112,7 @@ int fsadam_set_option(const char* name, int64_t value) {
         if (value < -1 || value > 65536) return fail(FSADAM_EINVAL, "lds_throttle must be -1 (per-mode default) or in [0, 65536] bytes");
         g_opt.lds_throttle = value;
     } else if (k == "xcd_remap") {
-        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "xcd_remap must be 0 or 1");
+        if (value < 0 || value > (1 << 28)) return fail(FSADAM_EINVAL, "xcd_remap must be 0 (off) or a run length in tiles");
         g_opt.xcd_remap = value;
     } else if (k == "grad_items") {
         if (value != 0 && value != 2 && value != 4 && value != 8) return fail(FSADAM_EINVAL, "grad_items must be 0 (automatic), 2, 4 or 8");

@@ -113,7 +113,8 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
  *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
  *                   per-mode default (13-16 KiB, default)
- *   "xcd_remap"     0/1: hand each XCD a contiguous eighth of the tiles (default 0)
+ *   "xcd_remap"     0: tiles in dispatch order (default); R > 0: regroup so that each of the eight XCDs
+ *                   takes runs of R consecutive tiles (a very large R gives each XCD one contiguous eighth)
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
  *                   4 for one that writes the gradients back (default 0)
  *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise

@@ -80,7 +80,7 @@ def test_options_roundtrip_and_validation():
         _cabi.set_option("groups", 2)
         _cabi.set_option("lds_throttle", 20480)
         assert (_cabi.get_option("block"), _cabi.get_option("groups"), _cabi.get_option("lds_throttle")) == (128, 2, 20480)
-        for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", 2), ("no_such_option", 1)):
+        for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", -1), ("no_such_option", 1)):
             with pytest.raises(_cabi.FsAdamError):
                 _cabi.set_option(name, bad)
     finally:
