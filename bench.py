@@ -219,9 +219,11 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32 arithmetic; fp16 params+grads, fp32 m/v" if args.mode == "MEMORY_EFFICIENT_MIXED_PRECISION" else "f32 arithmetic",
+        "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": workload, "numel": args.numel, "precision": args.mode, "tensors": 1, "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
+        "config": {"workload": workload, "numel": args.numel, "precision": args.mode, "tensors": 1,
+                   "storage": {"FULL_PRECISION": "p,g,m,v fp32", "MIXED_PRECISION": "p,m,v fp32; g, copy-out fp16",
+                               "MEMORY_EFFICIENT_MIXED_PRECISION": "p,g fp16; m,v fp32", "PURE_FP16": "p,g,m,v fp16"}[args.mode], "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
                    "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
                    "options": {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap")}},
         "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

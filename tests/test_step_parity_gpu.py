@@ -356,6 +356,34 @@ def test_c4_flat_shard_1p63e9_memory_efficient(oracle, cuda_device):
     _window_check(oracle, MEMEFF, before, sub, gs, [(0, cnt)], dict(DEFAULT, step=3, grad_scale=1024.0), "C4 misaligned view")
 
 
+def test_single_tensor_beyond_2_to_31_elements(oracle, cuda_device):
+    """One fp16 tensor of 2^31 + 2^20 + 5 elements (PURE_FP16, 17 GB): element counts and offsets are 64-bit
+    here (the reference keeps them in int, multi_tensor_apply.cuh:21,80).  Windows at the start, across
+    the 2^31 boundary and at the ragged end are re-computed by the oracle."""
+    from fairscale_amd import fused_adam_hip
+
+    n = (1 << 31) + (1 << 20) + 5
+    dev = cuda_device
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < n * 2 * 7:
+        pytest.skip("not enough device memory")
+    gen = torch.Generator(device=dev).manual_seed(7000)
+    p = torch.empty(n, device=dev, dtype=torch.float16).normal_(0, 0.02, generator=gen)
+    g = torch.empty(n, device=dev, dtype=torch.float16).normal_(0, 1e-3, generator=gen)
+    m = torch.zeros(n, device=dev, dtype=torch.float16)
+    v = torch.zeros(n, device=dev, dtype=torch.float16)
+    flag = torch.zeros(1, device=dev)
+    windows = [(0, 70000), ((1 << 31) - 40000, (1 << 31) + 40000), (n - 70000, n)] + _windows(n, 6, 65536, 7001)
+    before = {"p": p.clone(), "m": m.clone(), "v": v.clone()}
+    fused_adam_hip.adam(65536, None, [[p], [m], [v], [g]], 1e-3, 0.9, 0.999, 1e-8, 1.0, 65536.0, flag, 1, 1, 1, 0.01)
+    torch.cuda.synchronize()
+    kw = dict(DEFAULT, step=1, optim_scale=65536.0, decay=0.01)
+    _window_check(oracle, PURE16, before, {"p": p, "m": m, "v": v}, g, windows, kw, "beyond 2^31")
+    assert flag.item() == 0.0
+    # nothing outside the tensor was touched and nothing inside was skipped: every m is non-zero where g is
+    assert int((m[-(1 << 22):] != 0).sum().item()) == int((g[-(1 << 22):] != 0).sum().item())
+
+
 def test_c5_llama7b_pure_fp16_with_overflow_injection(oracle, cuda_device):
     """BASELINE config 5 at its real size: 291 tensors / 6.74e9 fp16 parameters, fp16 grads and state
     with optimizer-state scaling.  Step 1 is clean; in step 2 one gradient element in 10^6 is set to
