@@ -686,6 +686,7 @@ struct TableSlot {
     ChunkDesc* d_table = nullptr;
     ChunkDesc* h_table = nullptr;  // pinned
     hipEvent_t last_use = nullptr;
+    hipStream_t last_stream = nullptr;  // the stream last_use was recorded on
     bool used = false;
 };
 constexpr int kTableSlots = 3;
@@ -711,6 +712,19 @@ void slot_release(TableSlot& slot) {
     slot.d_table = slot.h_table = nullptr;
     slot.cap_descs = 0;
     slot.used = false;
+}
+
+// Work that reads a table slot (or a plan's partial sums) is ordered after the upload or launch that
+// touched it last when the caller moves to another stream; on one stream the order is already there.
+int order_after(hipEvent_t last_use, bool used, hipStream_t last_stream, hipStream_t stream) {
+    if (used && last_use && last_stream != stream) FS_HIP(hipStreamWaitEvent(stream, last_use, 0));
+    return FSADAM_OK;
+}
+int slot_mark(TableSlot& slot, hipStream_t stream) {
+    FS_HIP(hipEventRecord(slot.last_use, stream));
+    slot.last_stream = stream;
+    slot.used = true;
+    return FSADAM_OK;
 }
 
 void plan_release_buffers(FsAdamPlan* plan) {
@@ -834,8 +848,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     plan->rows.assign(tensors, tensors + n);
     if (n_descs > 0)
         FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
-    FS_HIP(hipEventRecord(slot.last_use, stream));
-    slot.used = true;
+    rc = slot_mark(slot, stream);
+    if (rc) return rc;
     plan->current = (plan->current + 1) % kTableSlots;
     plan->uploads += 1;
     return FSADAM_OK;
@@ -868,12 +882,13 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     const Layout& L = plan->layout;
     const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
     TableSlot& slot = plan->slots[plan->current];
-    int rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
+    int rc = order_after(slot.last_use, slot.used, slot.last_stream, stream);
+    if (rc) return rc;
+    rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
     if (rc) return rc;
     rc = launch_mode(plan->mode, slot.d_table + L.n_large_descs, L.n_small_descs, 0, plan->opt, s, found_inf, stream);
     if (rc) return rc;
-    FS_HIP(hipEventRecord(slot.last_use, stream));
-    return FSADAM_OK;
+    return slot_mark(slot, stream);
 }
 
 
@@ -891,6 +906,7 @@ struct GradPlan {
     GradPartial* d_partials = nullptr;  // [cap_partials] first stage, then [kReduceBlocks] second stage, then [1] total
     int64_t cap_partials = 0;
     hipEvent_t last_use = nullptr;
+    hipStream_t last_stream = nullptr;
     bool used = false;
     uint64_t lru = 0;
 };
@@ -1005,8 +1021,8 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     plan->rows.assign(grads, grads + n);
     if (n_descs > 0)
         FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
-    FS_HIP(hipEventRecord(slot.last_use, stream));
-    slot.used = true;
+    const int rc = slot_mark(slot, stream);
+    if (rc) return rc;
     plan->current = (plan->current + 1) % kTableSlots;
     return FSADAM_OK;
 }
@@ -1022,6 +1038,10 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     GradPartial* first = plan->d_partials;
     GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
     GradPartial* total = second + kReduceBlocks;
+    int rc = order_after(slot.last_use, slot.used, slot.last_stream, stream);
+    if (rc) return rc;
+    rc = order_after(plan->last_use, plan->used, plan->last_stream, stream);  // the partial sums are shared by every call
+    if (rc) return rc;
 #define FS_GRAD_LAUNCH(ITEMS)                                                                                                   \
     do {                                                                                                                        \
         if (large_blocks > 0)                                                                                                   \
@@ -1044,8 +1064,10 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total);
     hipLaunchKernelGGL(fsadam_grad_publish, dim3(1), dim3(64), 0, stream, total, (int)(sizeof(T) == 2), found_inf, sum_squares, abs_max);
     FS_HIP(hipGetLastError());
-    FS_HIP(hipEventRecord(slot.last_use, stream));
+    rc = slot_mark(slot, stream);
+    if (rc) return rc;
     FS_HIP(hipEventRecord(plan->last_use, stream));
+    plan->last_stream = stream;
     plan->used = true;
     return FSADAM_OK;
 }

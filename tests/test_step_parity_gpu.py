@@ -139,6 +139,34 @@ def test_misaligned_views(oracle, cuda_device, mode, which):
              grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
+def test_steps_alternating_between_streams(oracle, cuda_device):
+    """Every step runs on another stream than the one before.  In the first half the gradient tensors stay
+    where they are, so kernels on one stream read a table that was uploaded on another (the library
+    orders the two itself); in the second half they move, so each stream uploads its own table."""
+    from fairscale_amd import fused_adam_hip
+
+    host = C.Tensors(MEMEFF, [300_000, 5, 70_001, 1 << 18], 77)
+    dev = GpuList(host, cuda_device)
+    streams = [torch.cuda.Stream(device=cuda_device) for _ in range(3)]
+    flag = np.zeros(1, np.float32)
+    g = to_gpu(host.grads(1, g_std=1e-3, scale=1.0), cuda_device)
+    for step in range(1, 9):
+        grads = host.grads(step, g_std=1e-3, scale=1.0)
+        if step <= 4:
+            for dst, src in zip(g, grads):
+                dst.copy_(torch.from_numpy(src))
+        else:
+            g = to_gpu(grads, cuda_device)
+        torch.cuda.synchronize(cuda_device)  # the copies ran on the default stream, the last step on another
+        kw = dict(DEFAULT, step=step, grad_scale=1.0, optim_scale=1.0)
+        with torch.cuda.stream(streams[step % 3]):
+            fused_adam_hip.adam(65536, None, [dev.p, dev.m, dev.v, g], kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], 1.0, 1.0,
+                                dev.found_inf, step, 1, 1, 0.0)
+        oracle_step(oracle, host, grads, flag, **kw)
+        torch.cuda.synchronize(cuda_device)
+        compare(host, dev, f"alternating streams, step {step}")
+
+
 def test_zero_sized_tensors_in_list(oracle, cuda_device):
     run_case(oracle, cuda_device, FULL, [0, 5, 0, 0, 20000, 0], 2, 4300, DEFAULT)
 
