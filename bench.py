@@ -104,6 +104,45 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
     return out
 
 
+def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000):
+    """4096 fp32 tensors of log-uniform sizes (numel = max(1, round(2**U(0, 20)))), FULL_PRECISION with weight
+    decay and eps inside the square root: the list-handling case.  Host time per step (the calls return
+    without waiting), device time per step, and wall time of back-to-back steps."""
+    import random
+
+    from fairscale_amd import _rows
+    from fairscale_amd.optim import Adam, Precision
+
+    rng = random.Random(seed)
+    sizes = [max(1, round(2 ** rng.uniform(0.0, 20.0))) for _ in range(count)]
+    params = [torch.empty(n, device=device).normal_(0, 0.02).requires_grad_() for n in sizes]
+    for p in params:
+        p.grad = torch.empty_like(p).normal_(0, 1e-3)
+    opt = Adam(params, lr=1e-3, weight_decay=0.01, eps_inside_sqrt=True, precision=Precision.FULL_PRECISION)
+    for _ in range(warmup):
+        opt.step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        opt.step()
+    e1.record()
+    host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    total = sum(sizes)
+    plan = next(iter(opt._plans.values())).info()
+    out = {"tensors": count, "numel": total, "host_ms_per_step": host / steps * 1e3, "device_ms_per_step": e0.elapsed_time(e1) / steps,
+           "ms_per_step": wall / steps * 1e3, "params_per_s": total * steps / wall, "bytes_per_param": 28,
+           "achieved_gbs": total * 28 * steps / wall / 1e9, "frac_of_hbm_peak": total * 28 * steps / wall / 1e9 / HBM_PEAK_GBS,
+           "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "uploads": plan["uploads"],
+           "list_walk": "c++" if _rows.native is not None else "python"}
+    del opt, params
+    torch.cuda.empty_cache()
+    return out
+
+
 def measure_grad_pass(torch, numel, steps, warmup, device):
     """The pre-step gradient pass over the same shard's fp16 gradients: norms + overflow check only
     (2 B/param read) and with the unscale written back (2 B read + 2 B written)."""
@@ -205,6 +244,7 @@ def main():
                                    "achieved_gbs": r["achieved_gbs"], "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
     if not args.no_also:
         also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
+        also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device)
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"

@@ -1,7 +1,8 @@
-"""Compiles fsadam.hip into libfsadam.so next to this file (hipcc, gfx950 only).
+"""Compiles fsadam.hip into libfsadam.so next to this file (hipcc, gfx950 only), and the host-side
+helper tensor_rows.cpp into a CPython extension module (g++, against the installed torch).
 
-Usage: ``python -m fairscale_amd.csrc.build`` or ``build_library()``.  The library is kept in-tree so
-that a process which loads it shows it among its mapped files.
+Usage: ``python -m fairscale_amd.csrc.build``, or ``build_library()`` / ``build_rows_module()``.  Both
+files are kept in-tree so that a process which loads them shows them among its mapped files.
 """
 from __future__ import annotations
 
@@ -46,5 +47,43 @@ def build_library(verbose: bool = False) -> str:
     return LIBRARY
 
 
+ROWS_SOURCE = os.path.join(HERE, "tensor_rows.cpp")
+
+
+def rows_module_path() -> str:
+    import sysconfig
+
+    return os.path.join(HERE, "_tensor_rows" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_rows_module(verbose: bool = False) -> str:
+    """Always recompiles the list-gathering helper; returns the path of the extension module."""
+    import sysconfig
+
+    import pybind11
+    import torch
+    from torch.utils import cpp_extension
+
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("no C++ compiler found for the host-side helper")
+    out = rows_module_path()
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    for inc in [*cpp_extension.include_paths(), pybind11.get_include(), sysconfig.get_paths()["include"]]:
+        cmd += ["-isystem", inc]
+    for lib in cpp_extension.library_paths():
+        cmd += ["-L", lib, f"-Wl,-rpath,{lib}"]
+    cmd += ["-o", out + ".tmp", ROWS_SOURCE, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("compiling tensor_rows.cpp failed:\n" + " ".join(cmd) + "\n" + proc.stdout)
+    os.replace(out + ".tmp", out)
+    if verbose and proc.stdout.strip():
+        print(proc.stdout, file=sys.stderr)
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_rows_module(verbose=True))

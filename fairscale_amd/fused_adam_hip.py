@@ -13,9 +13,9 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
-from . import _cabi
+from . import _cabi, _rows
 
-__all__ = ["adam", "TensorListPlan", "mode_of_lists", "rows_of_lists"]
+__all__ = ["adam", "TensorListPlan", "mode_of_lists", "rows_of_lists", "checked_rows"]
 
 _ROW_WORDS = ctypes.sizeof(_cabi.FsAdamTensor) // 8
 assert _ROW_WORDS == 6, "FsAdamTensor is five pointers and one int64"
@@ -98,6 +98,39 @@ def rows_of_lists(tensor_lists: Sequence[Sequence[torch.Tensor]]) -> np.ndarray:
     return rows
 
 
+def mode_codes(mode: int) -> tuple:
+    """Element-type codes (0 float32, 1 float16) of the lists of a mode, for the C++ helper."""
+    return tuple(_rows.dtype_code(dt) for dt in _MODE_DTYPES[mode])
+
+
+def checked_rows(tensor_lists: Sequence[Sequence[torch.Tensor]], mode: int, rows: Optional[np.ndarray] = None):
+    """Validate the lists and return ``(rows, changed, device)``.
+
+    ``rows`` is a buffer of the right shape from an earlier call (or None): it is overwritten in place
+    and ``changed`` tells whether any word differs from what it held.  One C++ pass when the helper is
+    built; otherwise ``validate_lists`` + ``rows_of_lists``.
+    """
+    native = _rows.native
+    depth_ok = len(tensor_lists) == len(_MODE_DTYPES[mode])
+    if native is not None and depth_ok and len(tensor_lists[0]) > 0 and all(type(lst) is list for lst in tensor_lists):
+        n = len(tensor_lists[0])
+        first = tensor_lists[0][0]
+        if isinstance(first, torch.Tensor) and first.is_cuda:
+            fresh = rows is None or rows.shape != (n, _ROW_WORDS)
+            buf = np.zeros((n, _ROW_WORDS), dtype=np.int64) if fresh else rows
+            lists = tensor_lists if type(tensor_lists) is list else list(tensor_lists)
+            status = native.fill_rows(lists, mode_codes(mode), first.device.index, buf.ctypes.data, n)[0]
+            if status >= 0:
+                return buf, bool(fresh or status == native.CHANGED), first.device
+            if not fresh:
+                buf[:] = 0  # partly overwritten: whatever comes next counts as changed
+    # the Python walk raises the reference's messages for whatever the helper refused
+    device = validate_lists(tensor_lists, mode)
+    new = rows_of_lists(tensor_lists)
+    changed = rows is None or rows.shape != new.shape or not np.array_equal(rows, new)
+    return new, changed, device
+
+
 def _rows_ptr(rows: np.ndarray):
     return rows.ctypes.data_as(ctypes.POINTER(_cabi.FsAdamTensor))
 
@@ -118,12 +151,11 @@ def adam(chunk_size: int, noop_flag: Optional[torch.Tensor], tensor_lists: List[
     set to 1.0 when a stored fp16 ``m``/``v`` is non-finite (PURE_FP16 only) and never cleared.
     """
     precision = mode_of_lists(tensor_lists)
-    device = validate_lists(tensor_lists, precision)
+    rows, _, device = checked_rows(tensor_lists, precision)
     if found_inf is None or found_inf.dtype != torch.float32 or not found_inf.is_cuda or found_inf.numel() < 1:
         raise RuntimeError("found_inf must be a float32 device tensor with one element")
     if found_inf.device != device:
         raise RuntimeError("found_inf must live on the tensors' device")
-    rows = rows_of_lists(tensor_lists)
     L = _cabi.lib()
     with torch.cuda.device(device):
         _cabi.check(L.fsadam_step(_rows_ptr(rows), rows.shape[0], precision, lr, beta1, beta2, eps, grad_scale,
@@ -142,6 +174,7 @@ class TensorListPlan:
         self.precision = precision
         self.device = device
         self._rows: Optional[np.ndarray] = None
+        self._dirty = True  # the device table does not (yet) hold what _rows holds
         self._handle = ctypes.c_void_p()
         _cabi.check(_cabi.lib().fsadam_plan_create(precision, ctypes.byref(self._handle)))
 
@@ -163,18 +196,44 @@ class TensorListPlan:
         _cabi.check(_cabi.lib().fsadam_plan_info(self._handle, ctypes.byref(out)))
         return out.as_dict()
 
-    def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,
-             grad_scale: float, optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int,
-             bias_correction: int, decay: float) -> None:
+    def rows_buffer(self, n: int) -> np.ndarray:
+        """The (n, 6) int64 buffer the C++ walk fills in place; its contents mirror the device table
+        unless ``mark_dirty`` was called since."""
+        if self._rows is None or self._rows.shape != (n, _ROW_WORDS):
+            self._rows = np.zeros((n, _ROW_WORDS), dtype=np.int64)
+            self._dirty = True
+        return self._rows
+
+    def mark_dirty(self) -> None:
+        """The buffer was partly overwritten by a walk that stopped: send the next table regardless."""
+        self._dirty = True
+
+    def step_rows(self, changed: bool, lr: float, beta1: float, beta2: float, eps: float, grad_scale: float,
+                  optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int, bias_correction: int,
+                  decay: float) -> None:
+        """Step over the rows already written into ``rows_buffer`` (validated by whoever wrote them)."""
         L = _cabi.lib()
-        rows = rows_of_lists(tensor_lists)
+        rows = self._rows
         with torch.cuda.device(self.device):
             stream = _stream_handle(self.device)
-            if self._rows is None or rows.shape != self._rows.shape or not np.array_equal(rows, self._rows):
-                if validate_lists(tensor_lists, self.precision) != self.device:
-                    raise RuntimeError("tensor list moved to another device")
+            if changed or self._dirty:
                 _cabi.check(L.fsadam_plan_set_tensors(self._handle, _rows_ptr(rows), rows.shape[0], stream))
-                self._rows = rows
+                self._dirty = False
             flag = found_inf.data_ptr() if found_inf is not None else None
             _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, grad_scale, optim_scale, decay,
                                            int(step), int(eps_mode), int(bias_correction), flag, stream))
+
+    def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,
+             grad_scale: float, optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int,
+             bias_correction: int, decay: float) -> None:
+        try:
+            rows, changed, device = checked_rows(tensor_lists, self.precision, self._rows)
+        except Exception:
+            self._dirty = True
+            raise
+        if device != self.device:
+            self._dirty = True
+            raise RuntimeError("tensor list moved to another device")
+        self._rows = rows
+        self.step_rows(changed, lr, beta1, beta2, eps, grad_scale, optim_scale, found_inf, step, eps_mode,
+                       bias_correction, decay)

@@ -20,13 +20,15 @@ Deliberate differences, all supersets of the reference behaviour:
 """
 from __future__ import annotations
 
+from collections import defaultdict
 from enum import Enum, auto
+from operator import is_not
 from typing import Any, Callable, Dict, List, Optional, Tuple
 
 import torch
 
-from .. import _cabi
-from ..fused_adam_hip import TensorListPlan
+from .. import _cabi, _rows
+from ..fused_adam_hip import TensorListPlan, mode_codes
 
 _cabi.lib()  # loading the kernels is part of importing the optimizer: no library, no Adam
 
@@ -50,6 +52,41 @@ _NATIVE_MODE = {
 }
 
 _MAX_OPTIM_SCALE = 2 ** 16
+
+
+class _VersionedState(defaultdict):
+    """``optimizer.state`` that counts its own insertions and removals, so that the step can tell in
+    O(1) whether the per-parameter state dicts it collected earlier are still the ones in the map."""
+
+    version = 0
+
+    def __setitem__(self, key, value):
+        self.version += 1
+        super().__setitem__(key, value)
+
+    def __delitem__(self, key):
+        self.version += 1
+        super().__delitem__(key)
+
+    def pop(self, *args):
+        self.version += 1
+        return super().pop(*args)
+
+    def popitem(self):
+        self.version += 1
+        return super().popitem()
+
+    def clear(self):
+        self.version += 1
+        super().clear()
+
+    def update(self, *args, **kwargs):
+        self.version += 1
+        super().update(*args, **kwargs)
+
+    def setdefault(self, key, default=None):
+        self.version += 1
+        return super().setdefault(key, default)
 
 
 class Adam(torch.optim.Optimizer):
@@ -120,6 +157,7 @@ class Adam(torch.optim.Optimizer):
                  max_grad_norm=max_grad_norm),
         )
         self.eps_mode = 0 if eps_inside_sqrt else 1  # adam.py:117
+        self.state = _VersionedState(dict, self.state)
 
         self.fp32_param_groups: List[Any] = []
         if self.mixed_precision:
@@ -212,6 +250,8 @@ class Adam(torch.optim.Optimizer):
         Also (re)builds the group's fast-path cache when every parameter took part and shares one device."""
         mixed = self.mixed_precision
         copies = self.__dict__.get("_fp16_copies")
+        if type(self.state) is not _VersionedState:  # torch's load_state_dict / __setstate__ put a plain map back
+            self.state = _VersionedState(dict, self.state)
         state_map, optim_type = self.state, self.optim_type
         masters = self.fp32_param_groups[gi]["params"] if mixed else None
         batches: Dict[torch.device, List[List[torch.Tensor]]] = {}
@@ -249,25 +289,65 @@ class Adam(torch.optim.Optimizer):
         if len(states) == len(params) and len(batches) == 1:
             device, lists = next(iter(batches.items()))
             outs = lists[4] if depth == 5 else None
-            caches[gi] = (params, len(params), states, masters, outs, device)
+            caches[gi] = (params, tuple(params), states, masters, outs, device, state_map, state_map.version)
         else:
             caches.pop(gi, None)
         return batches, step_no
+
+    def _steady_group(self, gi: int, group: Dict[str, Any]):
+        """The cached view of a group whose every parameter took part in the last general walk, or None
+        when the parameter list, the state map or the fp32 master copies were replaced or edited since."""
+        cache = self.__dict__.get("_group_cache", {}).get(gi)
+        if cache is None:
+            return None
+        params, snapshot, states, masters, outs, device, state_map, version = cache
+        if group["params"] is not params or len(params) != len(snapshot) or len(snapshot) == 0:
+            return None
+        if self.state is not state_map or state_map.version != version:
+            return None
+        if masters is not None and (self.fp32_param_groups[gi]["params"] is not masters or len(masters) != len(snapshot)):
+            return None
+        return cache
+
+    def _gather_native(self, gi: int, group: Dict[str, Any], native_mode: int):
+        """The steady-state walk in one C++ loop (csrc/tensor_rows.cpp): gradients, state tensors,
+        checks, pointers and step counters.  Returns (plan, table_changed, step) or None when the
+        helper is not built or anything is out of the ordinary; the Python walks then decide."""
+        native = _rows.native
+        if native is None:
+            return None
+        cache = self._steady_group(gi, group)
+        if cache is None:
+            return None
+        params, snapshot, states, masters, outs, device, _, _ = cache
+        if device.type != "cuda":
+            return None
+        plan = self._plan_for(gi, device, native_mode)
+        codes = mode_codes(native_mode)
+        buf = plan.rows_buffer(len(snapshot))
+        status, _, _, step_no = native.gather(params, snapshot, masters, states, None if masters is not None else outs,
+                                               (codes[0], codes[1], codes[3]), device.index, buf.ctypes.data)
+        if status < 0:
+            plan.mark_dirty()
+            return None
+        return plan, status == native.CHANGED, step_no
+
+    def _plan_for(self, gi: int, device: torch.device, native_mode: int) -> TensorListPlan:
+        plan = self._plans.get((gi, device))
+        if plan is None:
+            plan = self._plans[(gi, device)] = TensorListPlan(native_mode, device)
+        return plan
 
     def _gather_fast(self, gi: int, group: Dict[str, Any]):
         """Same result as ``_gather`` for the steady state (every parameter of the group has a dense
         gradient and an initialised state, all on one device) without the per-parameter dictionary
         walk; returns (None, None) when that does not hold and the general walk must run."""
-        cache = self.__dict__.get("_group_cache", {}).get(gi)
+        cache = self._steady_group(gi, group)
         if cache is None:
             return None, None
-        params, count, states, masters, outs, device = cache
-        if group["params"] is not params or len(params) != count or count == 0:
-            return None, None
-        if self.state.get(params[-1]) is not states[-1] or self.state.get(params[0]) is not states[0]:
-            return None, None  # the state mapping was replaced (e.g. load_state_dict)
-        if masters is not None and (self.fp32_param_groups[gi]["params"] is not masters or len(masters) != count):
-            return None, None  # the fp32 master copies were rebuilt or replaced
+        params, snapshot, states, masters, outs, device, _, _ = cache
+        if any(map(is_not, params, snapshot)):
+            return None, None  # the list was edited in place: the collected states belong to other parameters
         grads = [p.grad for p in params]
         for g in grads:
             if g is None or g.is_sparse:
@@ -301,25 +381,35 @@ class Adam(torch.optim.Optimizer):
 
         for gi, group in enumerate(self.param_groups):
             beta1, beta2 = group["betas"]
-            batches, step_no = self._gather_fast(gi, group)
-            if batches is None:
-                batches, step_no = self._gather(gi, group)
-            if not batches:
-                # adam.py:256 indexes the first device of an empty dict
-                raise IndexError("list index out of range")
-
             flags: List[torch.Tensor] = []
-            for device, lists in batches.items():
+            bias_correction = 1 if group["bias_correction"] else 0
+            ready = self._gather_native(gi, group, native_mode)
+            if ready is not None:
+                plan, table_changed, step_no = ready
+                flag = None
+                if watch_overflow:
+                    flag = self._flag_for(plan.device)
+                    flag.zero_()
+                    flags.append(flag)
+                plan.step_rows(table_changed, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
+                               step_no, self.eps_mode, bias_correction, group["weight_decay"])
+                batches = None
+            else:
+                batches, step_no = self._gather_fast(gi, group)
+                if batches is None:
+                    batches, step_no = self._gather(gi, group)
+                if not batches:
+                    # adam.py:256 indexes the first device of an empty dict
+                    raise IndexError("list index out of range")
+            for device, lists in (batches or {}).items():
                 flag = None
                 if watch_overflow:
                     flag = self._flag_for(device)
                     flag.zero_()
                     flags.append(flag)
-                plan = self._plans.get((gi, device))
-                if plan is None:
-                    plan = self._plans[(gi, device)] = TensorListPlan(native_mode, device)
-                plan.step(lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
-                          step_no, self.eps_mode, 1 if group["bias_correction"] else 0, group["weight_decay"])
+                self._plan_for(gi, device, native_mode).step(
+                    lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag, step_no, self.eps_mode,
+                    bias_correction, group["weight_decay"])
 
             overflowed = bool(sum(f.item() for f in flags)) if flags else False  # adam.py:278
             if overflowed:
