@@ -21,8 +21,8 @@
 // The tensor list becomes a device-resident table of 64-byte chunk descriptors (five pointers
 // already advanced to the chunk, element count, alignment flag), uploaded once and reused every
 // step.  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
-// tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles, small tensors get
-// one descriptor per tile in a second launch, so ONE or TWO launches cover any number of tensors
+// tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles; small tensors get
+// one descriptor per tile, placed after the large ones, so ONE launch covers any number of tensors
 // (the reference needs a launch per 36 tensors / 320 chunks because its table travels by value in
 // the kernel arguments).  Tiles that are ragged (end of a tensor) or belong to a tensor with a
 // misaligned stream take an element-wise path with the same arithmetic.
@@ -53,7 +53,7 @@ namespace {
 
 constexpr int64_t kLargeThreshold = 131072;   // tensors with at least this many elements share descriptors
 constexpr int64_t kMinLargeChunk = 65536;     // elements per shared descriptor, lower bound
-constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room)
+constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room); option max_large_chunk lowers it
 
 struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points at the chunk's first element
     void* p;
@@ -269,11 +269,14 @@ __device__ __forceinline__ uint32_t tile_any(const ChunkDesc& d, uint32_t off, c
     return tile_elementwise<MODE, BLOCK, EPS_MODE, FAST_SCALES>(d, off, left < kTile ? left : kTile, s);
 }
 
-// One workgroup = one tile.  `log2k`: tiles per descriptor of this launch (0 for the small-tensor
-// launch).  `n_blocks`: tiles really launched for (the grid may be padded for the XCD remap).
+// One workgroup = one tile.  The first `n_large_blocks` tiles belong to the descriptors of large
+// tensors, 2^log2k tiles each; every tile after them has a descriptor of its own (small tensors),
+// stored behind the `n_large_descs` large ones.  `n_blocks`: tiles really launched for (the grid may
+// be padded for the XCD remap).
 template <int MODE, int BLOCK, int GROUPS>
-__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_blocks,
-                                                      uint32_t xcd_stride, StepScalars s, float* __restrict__ found_inf) {
+__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
+                                                      uint32_t n_large_descs, uint32_t n_blocks, uint32_t xcd_stride,
+                                                      StepScalars s, float* __restrict__ found_inf) {
     constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
 
     uint32_t block = blockIdx.x;
@@ -285,8 +288,9 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
         block = group * 8u * xcd_stride + (in_group & 7u) * xcd_stride + (in_group >> 3);
         if (block >= n_blocks) return;
     }
-    const uint32_t chunk = block >> log2k;
-    const uint32_t off = (block & ((1u << log2k) - 1u)) * kTile;
+    const bool large = block < n_large_blocks;  // uniform: scalar selects
+    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
+    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
     // The whole 64-byte descriptor in ONE scalar load (uniform address, constant address space), before
     // anything is tested: reading the count first and the pointers afterwards would put two memory
     // latencies in front of the first data load.
@@ -294,7 +298,7 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
     const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
         (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
     const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
-    if (off >= d.n) return;  // tile past the end of its tensor (large launch only)
+    if (off >= d.n) return;  // tile past the end of its tensor (large tensors only)
 
     uint32_t bad;
     if (s.eps_mode == 0) {
@@ -431,14 +435,16 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, floa
 }
 
 template <typename T, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, float inv_scale_value,
+__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
+                                                           uint32_t n_large_descs, float inv_scale_value,
                                                            const float* __restrict__ inv_scale_dev, int write_back,
                                                            GradPartial* __restrict__ partials) {
     static_assert(BLOCK == 64, "one wave per workgroup: the partial is reduced with wave shuffles only");
     constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
     const uint32_t block = blockIdx.x;
-    const uint32_t chunk = block >> log2k;
-    const uint32_t off = (block & ((1u << log2k) - 1u)) * kTile;
+    const bool large = block < n_large_blocks;  // uniform: scalar selects
+    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
+    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
     typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
     const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
         (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
@@ -563,6 +569,7 @@ struct Options {
     int64_t xcd_remap = 0;      // 0: tiles in dispatch order; R > 0: each XCD takes runs of R consecutive tiles
     int64_t grad_items = 0;     // gradient pass: 16-byte vectors per lane (2, 4 or 8; 0 = by kind of pass)
     int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
+    int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -666,7 +673,7 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
         }
     }
     // every large tensor spans at least two chunks, so the empty tiles after its end stay a small share
-    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
+    L.large_chunk_elems = std::min(opt.max_large_chunk, std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2)))));
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = tensors[t].numel;
         if (numel == 0) continue;
@@ -753,10 +760,11 @@ void fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t chunk_e
 }
 
 template <int MODE, int BLOCK, int GROUPS>
-int launch_tiles(const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s,
-                 float* found_inf, hipStream_t stream) {
-    if (n_descs == 0) return FSADAM_OK;
-    const int64_t n_blocks = n_descs << log2k;
+int launch_tiles(const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
+                 const StepScalars& s, float* found_inf, hipStream_t stream) {
+    const int64_t n_large_blocks = n_large_descs << log2k;
+    const int64_t n_blocks = n_large_blocks + n_small_descs;
+    if (n_blocks == 0) return FSADAM_OK;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
     uint32_t grid = (uint32_t)n_blocks, xcd_stride = 0;
     if (opt.xcd_remap) {  // value = tiles per run; 1 would be the identity
@@ -764,32 +772,35 @@ int launch_tiles(const ChunkDesc* table, int64_t n_descs, int log2k, const Optio
         grid = (uint32_t)(ceil_div(n_blocks, 8 * (int64_t)xcd_stride) * 8 * xcd_stride);
     }
     hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table,
-                       (uint32_t)log2k, (uint32_t)n_blocks, xcd_stride, s, found_inf);
+                       (uint32_t)log2k, (uint32_t)n_large_blocks, (uint32_t)n_large_descs, (uint32_t)n_blocks, xcd_stride, s,
+                       found_inf);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
 
 template <int MODE>
-int launch_shape(const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s, float* found_inf,
-                 hipStream_t stream) {
-#define FS_CASE(B, G) \
-    if (opt.block == B && opt.groups == G) return launch_tiles<MODE, B, G>(table, n_descs, log2k, opt, s, found_inf, stream)
+int launch_shape(const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
+                 const StepScalars& s, float* found_inf, hipStream_t stream) {
+#define FS_CASE(B, G)                      \
+    if (opt.block == B && opt.groups == G) \
+    return launch_tiles<MODE, B, G>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream)
     FS_CASE(64, 1); FS_CASE(64, 2); FS_CASE(128, 1); FS_CASE(128, 2); FS_CASE(256, 1); FS_CASE(256, 2);
 #undef FS_CASE
     return fail(FSADAM_EINVAL, "unsupported block/groups combination");
 }
 
-int launch_mode(int mode, const ChunkDesc* table, int64_t n_descs, int log2k, const Options& opt, const StepScalars& s,
-                float* found_inf, hipStream_t stream) {
+int launch_mode(int mode, const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
+                const StepScalars& s, float* found_inf, hipStream_t stream) {
+#define FS_MODE(M) \
+    case M: return launch_shape<M>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream)
     switch (mode) {
-        case FSADAM_FULL_PRECISION: return launch_shape<FSADAM_FULL_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
-        case FSADAM_MIXED_PRECISION: return launch_shape<FSADAM_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
-        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION:
-            return launch_shape<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION>(table, n_descs, log2k, opt, s, found_inf, stream);
-        case FSADAM_FULL_PRECISION_FP16_COPY:
-            return launch_shape<FSADAM_FULL_PRECISION_FP16_COPY>(table, n_descs, log2k, opt, s, found_inf, stream);
-        default: return launch_shape<FSADAM_PURE_FP16>(table, n_descs, log2k, opt, s, found_inf, stream);
+        FS_MODE(FSADAM_FULL_PRECISION);
+        FS_MODE(FSADAM_MIXED_PRECISION);
+        FS_MODE(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION);
+        FS_MODE(FSADAM_FULL_PRECISION_FP16_COPY);
+        default: return launch_shape<FSADAM_PURE_FP16>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream);
     }
+#undef FS_MODE
 }
 
 int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, hipStream_t stream) {
@@ -808,7 +819,7 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
     const Layout L = compute_layout(tensors, n, plan->mode, plan->opt);
     const int64_t n_descs = L.n_large_descs + L.n_small_descs;
-    if (L.n_large_descs * (L.large_chunk_elems / L.tile_elems) > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0)
+    if (L.n_large_descs * (L.large_chunk_elems / L.tile_elems) + L.n_small_descs > 0x7ffffff0)
         return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
     // next slot of the ring; it may still be read by the step that used it last
@@ -829,7 +840,7 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
         }
         slot.cap_descs = cap;
     }
-    // large tensors first (one launch), then small ones (second launch)
+    // descriptors of large tensors first, then those of small ones: one launch covers both
     ChunkDesc* large = slot.h_table;
     ChunkDesc* small = slot.h_table + L.n_large_descs;
     for (int64_t t = 0; t < n; ++t) {
@@ -884,9 +895,7 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     TableSlot& slot = plan->slots[plan->current];
     int rc = order_after(slot.last_use, slot.used, slot.last_stream, stream);
     if (rc) return rc;
-    rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, log2k, plan->opt, s, found_inf, stream);
-    if (rc) return rc;
-    rc = launch_mode(plan->mode, slot.d_table + L.n_large_descs, L.n_small_descs, 0, plan->opt, s, found_inf, stream);
+    rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, L.n_small_descs, log2k, plan->opt, s, found_inf, stream);
     if (rc) return rc;
     return slot_mark(slot, stream);
 }
@@ -899,6 +908,7 @@ struct GradPlan {
     int dtype = 0;
     int64_t items = 4;
     int64_t lds_throttle = 0;
+    int64_t max_large_chunk = kMaxLargeChunk;
     std::vector<FsGradTensor> rows;
     Layout layout;
     TableSlot slots[kTableSlots];
@@ -916,7 +926,7 @@ constexpr int kReduceBlocks = 512;
 int grad_elem_size(int dtype) { return dtype == FSADAM_GRAD_F16 ? 2 : 4; }
 int64_t grad_tile_elems(int dtype, int64_t items) { return 64 * (16 / grad_elem_size(dtype)) * items; }
 
-Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items) {
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk) {
     Layout L;
     L.tile_elems = grad_tile_elems(dtype, items);
     int64_t min_large = 0;
@@ -932,7 +942,7 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
             L.n_small += 1;
         }
     }
-    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
+    L.large_chunk_elems = std::min(max_large_chunk, std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2)))));
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = grads[t].numel;
         if (numel == 0) continue;
@@ -955,17 +965,18 @@ void grad_plan_free(GradPlan* plan) {
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
-void grad_shape(bool writes, int64_t* items, int64_t* lds) {
+void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    *max_large_chunk = g_opt.max_large_chunk;
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
     *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 13312 : 16384);
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
-    const Layout L = grad_layout(grads, n, plan->dtype, plan->items);
+    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk);
     const int64_t k = L.large_chunk_elems / L.tile_elems;
     const int64_t n_blocks = L.n_large_descs * k + L.n_small_descs;
-    if (L.n_large_descs * k > 0x7ffffff0 || L.n_small_descs > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
+    if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
     const int64_t n_descs = L.n_large_descs + L.n_small_descs;
     TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
     if (!slot.last_use) FS_HIP(hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming));
@@ -1042,14 +1053,12 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     if (rc) return rc;
     rc = order_after(plan->last_use, plan->used, plan->last_stream, stream);  // the partial sums are shared by every call
     if (rc) return rc;
-#define FS_GRAD_LAUNCH(ITEMS)                                                                                                   \
-    do {                                                                                                                        \
-        if (large_blocks > 0)                                                                                                   \
-            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)large_blocks), dim3(64), lds, stream,          \
-                               slot.d_table, (uint32_t)log2k, inv_scale, inv_scale_dev, write_back, first);                    \
-        if (L.n_small_descs > 0)                                                                                                \
-            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)L.n_small_descs), dim3(64), lds, stream,       \
-                               slot.d_table + L.n_large_descs, 0u, inv_scale, inv_scale_dev, write_back, first + large_blocks); \
+#define FS_GRAD_LAUNCH(ITEMS)                                                                                               \
+    do {                                                                                                                    \
+        if (n_blocks > 0)                                                                                                   \
+            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)n_blocks), dim3(64), lds, stream,          \
+                               slot.d_table, (uint32_t)log2k, (uint32_t)large_blocks, (uint32_t)L.n_large_descs, inv_scale, \
+                               inv_scale_dev, write_back, first);                                                           \
     } while (0)
     const size_t lds = (size_t)plan->lds_throttle;
     if (plan->items == 2) FS_GRAD_LAUNCH(2);
@@ -1097,7 +1106,8 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
 }
 
 bool same_options(const Options& a, const Options& b) {
-    return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap;
+    return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap &&
+           a.max_large_chunk == b.max_large_chunk;
 }
 
 }  // namespace
@@ -1136,6 +1146,10 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "xcd_remap") {
         if (value < 0 || value > (1 << 28)) return fail(FSADAM_EINVAL, "xcd_remap must be 0 (off) or a run length in tiles");
         g_opt.xcd_remap = value;
+    } else if (k == "max_large_chunk") {
+        if (value < 4096 || value > kMaxLargeChunk || (value & (value - 1)) != 0)
+            return fail(FSADAM_EINVAL, "max_large_chunk must be a power of two in [4096, 2^24] elements");
+        g_opt.max_large_chunk = value;
     } else if (k == "grad_items") {
         if (value != 0 && value != 2 && value != 4 && value != 8) return fail(FSADAM_EINVAL, "grad_items must be 0 (automatic), 2, 4 or 8");
         g_opt.grad_items = value;
@@ -1156,6 +1170,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "groups") *value = g_opt.groups;
     else if (k == "lds_throttle") *value = g_opt.lds_throttle;
     else if (k == "xcd_remap") *value = g_opt.xcd_remap;
+    else if (k == "max_large_chunk") *value = g_opt.max_large_chunk;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
@@ -1225,7 +1240,7 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
     out->n_descriptors = L.n_large_descs + L.n_small_descs;
     out->n_vector_tensors = L.n_vector;
     out->n_scalar_tensors = L.n_scalar;
-    out->n_launches = (L.n_large_descs > 0) + (L.n_small_descs > 0);
+    out->n_launches = (L.n_large_descs + L.n_small_descs) > 0 ? 1 : 0;
     out->grid = L.tile_elems ? L.n_large_descs * (L.large_chunk_elems / L.tile_elems) + L.n_small_descs : 0;
     out->block = plan->opt.block;
     out->lds_throttle = plan->opt.lds_throttle;
@@ -1302,14 +1317,14 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    int64_t cur_items, cur_lds;
-    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds);
+    int64_t cur_items, cur_lds, cur_chunk;
+    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->max_large_chunk == cur_chunk && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -1332,6 +1347,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         }
         victim->items = cur_items;
         victim->lds_throttle = cur_lds;
+        victim->max_large_chunk = cur_chunk;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;
