@@ -243,12 +243,52 @@ py::tuple gather(py::list params, py::tuple snapshot, py::object masters, py::li
     return as_tuple(r, py::reinterpret_steal<py::object>(last));
 }
 
+// Gradients of one pass (include/fsadam.h: FsGradTensor rows, n x 2 int64: pointer, numel): dense,
+// contiguous, one dtype, one device.
+//
+// fill_grad_rows(grads, dtype_code, device_index, rows_address) -> (status, 3, index, None)
+py::tuple fill_grad_rows(py::list grads, int dtype_code, int device, uintptr_t rows_address) {
+    Result r;
+    r.list = 3;
+    const int64_t n = PyList_GET_SIZE(grads.ptr());
+    if (n < 1 || !rows_address) {
+        r.status = kLength;
+        return as_tuple(r);
+    }
+    const c10::ScalarType dtype = dtype_of_code(dtype_code);
+    int64_t* rows = reinterpret_cast<int64_t*>(rows_address);
+    try {
+        for (int64_t t = 0; t < n; ++t) {
+            const at::Tensor* g = plain_tensor(PyList_GET_ITEM(grads.ptr(), t));
+            r.index = t;
+            if (!g) {
+                r.status = kNotTensor;
+                return as_tuple(r);
+            }
+            const int bad = check_tensor(*g, dtype, device, g->numel());
+            if (bad) {
+                r.status = bad;
+                return as_tuple(r);
+            }
+            rows[t * 2 + 0] = reinterpret_cast<int64_t>(g->data_ptr());
+            rows[t * 2 + 1] = g->numel();
+        }
+    } catch (const std::exception& e) {
+        r.status = kError;
+        return as_tuple(r, py::str(e.what()));
+    }
+    r.index = -1;
+    r.status = kUnchanged;
+    return as_tuple(r);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_tensor_rows, m) {
     m.doc() = "Tensor lists -> FsAdamTensor rows for libfsadam (pointers and metadata only)";
     m.def("fill_rows", &fill_rows);
     m.def("gather", &gather);
+    m.def("fill_grad_rows", &fill_grad_rows);
     m.attr("UNCHANGED") = (int)kUnchanged;
     m.attr("CHANGED") = (int)kChanged;
     m.attr("NOT_TENSOR") = (int)kNotTensor;

@@ -22,7 +22,7 @@ from typing import Dict, Iterable, List, NamedTuple, Optional, Sequence, Tuple, 
 import numpy as np
 import torch
 
-from . import _cabi
+from . import _cabi, _rows
 
 __all__ = ["GradStats", "grad_pass", "calc_grad_norm", "clip_grad_norm_"]
 
@@ -56,11 +56,22 @@ def grad_pass(grads: Sequence[torch.Tensor], inv_scale: Union[float, torch.Tenso
     device, dtype = grads[0].device, grads[0].dtype
     if dtype not in _DTYPE_CODE:
         raise RuntimeError(f"gradients must be float16 or float32, got {dtype}")
-    for g in grads:
-        if g.device != device or g.dtype != dtype:
-            raise RuntimeError("gradients of one pass must share device and dtype")
-        if not g.is_cuda or g.is_sparse or not g.is_contiguous():
-            raise RuntimeError("gradients must be dense, contiguous device tensors")
+    rows = np.empty((len(grads), 2), dtype=np.int64)
+    native = _rows.native
+    checked = False
+    if native is not None and device.type == "cuda":
+        # one C++ loop: layout, contiguity, device, dtype, pointer, numel
+        status = native.fill_grad_rows(grads if type(grads) is list else list(grads), _rows.dtype_code(dtype), device.index,
+                                       rows.ctypes.data)[0]
+        checked = status >= 0
+    if not checked:  # also names what the helper refused
+        for g in grads:
+            if g.device != device or g.dtype != dtype:
+                raise RuntimeError("gradients of one pass must share device and dtype")
+            if not g.is_cuda or g.is_sparse or not g.is_contiguous():
+                raise RuntimeError("gradients must be dense, contiguous device tensors")
+        rows[:, 0] = list(map(torch.Tensor.data_ptr, grads))
+        rows[:, 1] = list(map(torch.Tensor.numel, grads))
     if found_inf is None:
         found_inf = torch.zeros(1, dtype=torch.float32, device=device)
     elif found_inf.dtype != torch.float32 or found_inf.device != device or found_inf.numel() != 1:
@@ -74,9 +85,6 @@ def grad_pass(grads: Sequence[torch.Tensor], inv_scale: Union[float, torch.Tenso
         scale_value = float(inv_scale)
     sum_squares = torch.empty(1, dtype=torch.float64, device=device)
     abs_max = torch.empty(1, dtype=torch.float32, device=device)
-    rows = np.empty((len(grads), 2), dtype=np.int64)
-    rows[:, 0] = list(map(torch.Tensor.data_ptr, grads))
-    rows[:, 1] = list(map(torch.Tensor.numel, grads))
     with torch.cuda.device(device):
         _cabi.check(_cabi.lib().fsadam_grad_pass(
             rows.ctypes.data_as(ctypes.POINTER(_cabi.FsGradTensor)), len(grads), _DTYPE_CODE[dtype], scale_value, scale_ptr,
@@ -102,11 +110,12 @@ def calc_grad_norm(parameters: Union[torch.Tensor, Iterable[torch.nn.Parameter]]
     if len(params) == 0:
         return torch.tensor(0.0)
     p = float(p)
-    grads = [par.grad.detach() for par in params]
-    if p not in (2.0, inf) or not all(supported(g) for g in grads):
-        if p == inf:
-            return max(g.abs().max() for g in grads)
-        return torch.norm(torch.stack([torch.norm(g, p, dtype=torch.float32) for g in grads]), p).to(dtype=params[0].dtype)
+    grads = [par.grad for par in params]  # only read here; nothing below records autograd history
+    if p not in (2.0, inf) or not all(map(supported, grads)):
+        with torch.no_grad():
+            if p == inf:
+                return max(g.abs().max() for g in grads)
+            return torch.norm(torch.stack([torch.norm(g, p, dtype=torch.float32) for g in grads]), p).to(dtype=params[0].dtype)
     first = grads[0].device
     stats = [grad_pass(group, 1.0, write_back=False) for group in _by_device_and_dtype(grads).values()]
     if p == inf:
@@ -142,12 +151,13 @@ def clip_grad_norm_(parameters: Union[torch.Tensor, Iterable[torch.nn.Parameter]
     if fold:
         return total_norm, (1.0 / float(clip_coef)) if clipping else 1.0
     if clipping:
-        grads = [par.grad.detach() for par in params]
+        grads = [par.grad for par in params]
         fast = [g for g in grads if supported(g)]
         for group in _by_device_and_dtype(fast).values():
             coef = clip_coef.to(device=group[0].device, dtype=torch.float32).reshape(1)
             grad_pass(group, coef, write_back=True)
-        for g in grads:
-            if not supported(g):
-                g.mul_(clip_coef.to(g.device))
+        with torch.no_grad():
+            for g in grads:
+                if not supported(g):
+                    g.mul_(clip_coef.to(g.device))
     return total_norm

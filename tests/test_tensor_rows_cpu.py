@@ -210,3 +210,17 @@ def test_tensor_subclasses_are_left_to_the_python_walk():
     lists[0][1] = torch.zeros(4).as_subclass(Tagged)
     rows = np.zeros((2, 6), np.int64)
     assert fill(lists, (F32,) * 4, rows)[:3] == (native.NOT_TENSOR, 0, 1)
+
+
+def test_fill_grad_rows():
+    grads = [torch.zeros(n, dtype=torch.float16) for n in (5, 0, 70001)]
+    rows = np.zeros((3, 2), np.int64)
+    assert native.fill_grad_rows(grads, F16, -1, rows.ctypes.data) == (native.UNCHANGED, 3, -1, None)
+    assert rows[:, 0].tolist() == [g.data_ptr() for g in grads] and rows[:, 1].tolist() == [5, 0, 70001]
+    assert native.fill_grad_rows(grads, F32, -1, rows.ctypes.data)[:3] == (native.DTYPE, 3, 0)
+    grads[2] = torch.zeros(140002, dtype=torch.float16)[::2]
+    assert native.fill_grad_rows(grads, F16, -1, rows.ctypes.data)[:3] == (native.NOT_CONTIGUOUS, 3, 2)
+    grads[2] = torch.zeros(4, dtype=torch.float16).to_sparse()
+    assert native.fill_grad_rows(grads, F16, -1, rows.ctypes.data)[:3] == (native.SPARSE, 3, 2)
+    assert native.fill_grad_rows(grads[:2], F16, 0, rows.ctypes.data)[:3] == (native.NOT_CUDA, 3, 0)
+    assert native.fill_grad_rows([], F16, -1, rows.ctypes.data)[0] == native.LENGTH
