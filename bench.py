@@ -6,8 +6,10 @@
 Workload (BASELINE.json configs[3], the one the metric is quoted on): a single rank's OSS shard of a
 13B model -- one contiguous buffer of 1.63e9 parameters, MEMORY_EFFICIENT_MIXED_PRECISION (fp16
 params and grads, fp32 m/v, grads scaled by 1024).  A "step" is one ``Adam.step()`` over that shard
-with everything resident in HBM.  Prints ONE JSON line; the same shard stepped in MIXED_PRECISION
-(fp32 master + fp16 grads + fp16 copy-out, 28 B/param) is reported under "also".
+with everything resident in HBM.  Prints ONE JSON line; under "also": the same number of parameters
+stepped in the other three dtype combinations (MIXED_PRECISION = fp32 master + fp16 grads + fp16
+copy-out, 28 B/param; FULL_PRECISION 28; PURE_FP16 14), the pre-step gradient pass over the shard's
+fp16 gradients, and a list of 4096 ragged fp32 tensors (host time and device time per step).
 
 "roofline" prices the dominant kernel against 8 TB/s of HBM: algorithmic bytes per launch (22 B per
 parameter in this mode: reads p16,g16,m32,v32, writes p16,m32,v32) over the kernel's average duration
@@ -38,7 +40,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--numel", type=int, default=SHARD_NUMEL, help="parameters in the flat shard")
     ap.add_argument("--mode", default="MEMORY_EFFICIENT_MIXED_PRECISION", choices=list(BYTES_PER_PARAM))
-    ap.add_argument("--no-also", action="store_true", help="skip the secondary MIXED_PRECISION measurement")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary measurements (other dtype combinations, gradient pass, ragged list)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-numel", type=int, default=1 << 26, help="sample size of the CPU baseline")
     ap.add_argument("--calib-copy-bytes", type=int, default=0,
@@ -238,10 +240,15 @@ def main():
 
     main_res = measure_gpu(torch, args.mode, args.numel, args.steps, args.warmup, device)
     also = {}
-    if not args.no_also and args.mode != "MIXED_PRECISION":
-        r = measure_gpu(torch, "MIXED_PRECISION", args.numel, args.steps, args.warmup, device)
-        also["MIXED_PRECISION"] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
-                                   "achieved_gbs": r["achieved_gbs"], "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
+    if not args.no_also:
+        # the other three dtype combinations on the same number of parameters
+        for mode in ("MIXED_PRECISION", "FULL_PRECISION", "PURE_FP16", "MEMORY_EFFICIENT_MIXED_PRECISION"):
+            if mode == args.mode:
+                continue
+            r = measure_gpu(torch, mode, args.numel, args.steps, args.warmup, device)
+            also[mode] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
+                          "bytes_per_param": r["bytes_per_param"], "achieved_gbs": r["achieved_gbs"],
+                          "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
     if not args.no_also:
         also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
         also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device)
