@@ -1,0 +1,172 @@
+/*
+ * The C ABI of include/fsadam.h used the way a non-Python host would: plain C, the HIP runtime for
+ * device memory, no torch in the process.  Every precision mode steps a small ragged tensor list
+ * three times through fsadam_step (the drop-in for fairscale.fused_adam_cuda.adam,
+ * fairscale/clib/fused_adam_cuda/fused_adam_cuda.cpp:4-8) and once more through a plan; the results
+ * are compared bit for bit with the CPU oracle (test infrastructure, oracle/adam_oracle.c) linked
+ * into this program.  Prints one line per mode and exits 0 when everything is identical.
+ *
+ * Built by tests/cabi_driver/Makefile (hipcc as the C compiler driver for the runtime's include and
+ * library paths); run by tests/test_cabi_driver_gpu.py.
+ */
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "fsadam.h"
+
+/* oracle/adam_oracle.c */
+uint16_t oracle_float_to_half(float f);
+int fsadam_oracle_step(int mode, void* p, void* m, void* v, const void* g, void* p_copy, int64_t n, float lr, float b1,
+                       float b2, float eps, float grad_scale, float optim_scale, float decay, int step, int eps_mode,
+                       int bias_correction, float* found_inf);
+
+#define CHECK_HIP(call)                                                                  \
+    do {                                                                                 \
+        hipError_t e_ = (call);                                                          \
+        if (e_ != hipSuccess) {                                                          \
+            fprintf(stderr, "%s: %s\n", #call, hipGetErrorString(e_));                   \
+            return 2;                                                                    \
+        }                                                                                \
+    } while (0)
+#define CHECK_FS(call)                                                                   \
+    do {                                                                                 \
+        int rc_ = (call);                                                                \
+        if (rc_ != FSADAM_OK) {                                                          \
+            fprintf(stderr, "%s -> %d: %s\n", #call, rc_, fsadam_last_error());          \
+            return 3;                                                                    \
+        }                                                                                \
+    } while (0)
+
+enum { N_TENSORS = 7, N_STEPS = 4 };
+static const int64_t kSizes[N_TENSORS] = {1, 255, 256, 257, 0, 70001, 300000};
+
+static uint64_t g_state = 0x9e3779b97f4a7c15ull;
+static float uniform_pm1(void) { /* xorshift64*: deterministic, in (-1, 1) */
+    g_state ^= g_state >> 12;
+    g_state ^= g_state << 25;
+    g_state ^= g_state >> 27;
+    const uint64_t r = g_state * 0x2545f4914f6cdd1dull;
+    return (float)((double)(r >> 11) / 9007199254740992.0 * 2.0 - 1.0);
+}
+
+static int elem_size(int is_half) { return is_half ? 2 : 4; }
+
+static void fill(void* dst, int64_t n, int is_half, float scale) {
+    for (int64_t i = 0; i < n; ++i) {
+        const float x = uniform_pm1() * scale;
+        if (is_half) ((uint16_t*)dst)[i] = oracle_float_to_half(x);
+        else ((float*)dst)[i] = x;
+    }
+}
+
+typedef struct {
+    void *h[5], *d[5]; /* p, m, v, g, p_copy: host (oracle) and device copies */
+} Streams;
+
+static int run_mode(int mode, const char* name) {
+    const int p_half = (mode == FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION || mode == FSADAM_PURE_FP16);
+    const int s_half = (mode == FSADAM_PURE_FP16);
+    const int g_half = !(mode == FSADAM_FULL_PRECISION || mode == FSADAM_FULL_PRECISION_FP16_COPY);
+    const int has_copy = (mode == FSADAM_MIXED_PRECISION || mode == FSADAM_FULL_PRECISION_FP16_COPY);
+    const int half_of[5] = {p_half, s_half, s_half, g_half, 1};
+    const float optim_scale = mode == FSADAM_PURE_FP16 ? 65536.0f : 1.0f;
+    const float grad_scale = g_half ? 128.0f : 1.0f;
+    Streams t[N_TENSORS];
+    FsAdamTensor rows[N_TENSORS];
+    float* d_flag = NULL;
+    float h_flag = 0.0f, oracle_flag = 0.0f;
+    hipStream_t stream;
+    CHECK_HIP(hipStreamCreate(&stream));
+    CHECK_HIP(hipMalloc((void**)&d_flag, sizeof(float)));
+    CHECK_HIP(hipMemset(d_flag, 0, sizeof(float)));
+    memset(t, 0, sizeof(t));
+    for (int i = 0; i < N_TENSORS; ++i) {
+        const int64_t n = kSizes[i];
+        for (int s = 0; s < 5; ++s) {
+            if (s == 4 && !has_copy) continue;
+            const size_t bytes = (size_t)(n > 0 ? n : 1) * elem_size(half_of[s]);
+            t[i].h[s] = calloc(1, bytes);
+            CHECK_HIP(hipMalloc(&t[i].d[s], bytes));
+            if (s == 0) fill(t[i].h[s], n, half_of[s], 0.02f);
+            CHECK_HIP(hipMemcpy(t[i].d[s], t[i].h[s], bytes, hipMemcpyHostToDevice));
+        }
+        rows[i].p = t[i].d[0];
+        rows[i].m = t[i].d[1];
+        rows[i].v = t[i].d[2];
+        rows[i].g = t[i].d[3];
+        rows[i].p_copy = t[i].d[4];
+        rows[i].numel = n;
+    }
+    FsAdamPlan* plan = NULL;
+    CHECK_FS(fsadam_plan_create(mode, &plan));
+    for (int step = 1; step <= N_STEPS; ++step) {
+        for (int i = 0; i < N_TENSORS; ++i) { /* fresh gradients, same on both sides */
+            fill(t[i].h[3], kSizes[i], g_half, 1e-3f * grad_scale);
+            CHECK_HIP(hipMemcpyAsync(t[i].d[3], t[i].h[3], (size_t)kSizes[i] * elem_size(g_half), hipMemcpyHostToDevice, stream));
+        }
+        if (step < N_STEPS) {
+            CHECK_FS(fsadam_step(rows, N_TENSORS, mode, 1e-3f, 0.9f, 0.999f, 1e-8f, grad_scale, optim_scale, 0.01f, step,
+                                 FSADAM_EPS_OUTSIDE_SQRT, 1, d_flag, stream));
+        } else { /* the last step through an explicit plan */
+            CHECK_FS(fsadam_plan_set_tensors(plan, rows, N_TENSORS, stream));
+            CHECK_FS(fsadam_plan_step(plan, 1e-3f, 0.9f, 0.999f, 1e-8f, grad_scale, optim_scale, 0.01f, step,
+                                      FSADAM_EPS_OUTSIDE_SQRT, 1, d_flag, stream));
+        }
+        for (int i = 0; i < N_TENSORS; ++i) {
+            if (kSizes[i] == 0) continue;
+            if (fsadam_oracle_step(mode, t[i].h[0], t[i].h[1], t[i].h[2], t[i].h[3], t[i].h[4], kSizes[i], 1e-3f, 0.9f, 0.999f,
+                                   1e-8f, grad_scale, optim_scale, 0.01f, step, FSADAM_EPS_OUTSIDE_SQRT, 1, &oracle_flag) != 0) {
+                fprintf(stderr, "oracle refused mode %d\n", mode);
+                return 4;
+            }
+        }
+        CHECK_HIP(hipStreamSynchronize(stream)); /* the next step overwrites the gradients */
+    }
+    int64_t different = 0, compared = 0;
+    for (int i = 0; i < N_TENSORS; ++i) {
+        for (int s = 0; s < 5; ++s) {
+            if (s == 3 || !t[i].d[s] || kSizes[i] == 0) continue;
+            const size_t bytes = (size_t)kSizes[i] * elem_size(half_of[s]);
+            unsigned char* got = (unsigned char*)malloc(bytes);
+            CHECK_HIP(hipMemcpy(got, t[i].d[s], bytes, hipMemcpyDeviceToHost));
+            for (size_t b = 0; b < bytes; ++b) different += got[b] != ((unsigned char*)t[i].h[s])[b];
+            compared += (int64_t)bytes;
+            free(got);
+        }
+    }
+    CHECK_HIP(hipMemcpy(&h_flag, d_flag, sizeof(float), hipMemcpyDeviceToHost));
+    FsAdamPlanInfo info;
+    CHECK_FS(fsadam_plan_info(plan, &info));
+    CHECK_FS(fsadam_plan_destroy(plan));
+    for (int i = 0; i < N_TENSORS; ++i)
+        for (int s = 0; s < 5; ++s) {
+            if (t[i].d[s]) CHECK_HIP(hipFree(t[i].d[s]));
+            free(t[i].h[s]);
+        }
+    CHECK_HIP(hipFree(d_flag));
+    CHECK_HIP(hipStreamDestroy(stream));
+    printf("%-40s %lld bytes compared, %lld differ, flag %g (oracle %g), %lld descriptors, %lld launch(es)\n", name,
+           (long long)compared, (long long)different, h_flag, oracle_flag, (long long)info.n_descriptors, (long long)info.n_launches);
+    return (different == 0 && h_flag == oracle_flag) ? 0 : 1;
+}
+
+int main(void) {
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev < 1) {
+        fprintf(stderr, "no GPU\n");
+        return 2;
+    }
+    printf("libfsadam ABI %d\n", fsadam_version());
+    int bad = 0;
+    bad |= run_mode(FSADAM_FULL_PRECISION, "FULL_PRECISION");
+    bad |= run_mode(FSADAM_MIXED_PRECISION, "MIXED_PRECISION");
+    bad |= run_mode(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION, "MEMORY_EFFICIENT_MIXED_PRECISION");
+    bad |= run_mode(FSADAM_PURE_FP16, "PURE_FP16");
+    bad |= run_mode(FSADAM_FULL_PRECISION_FP16_COPY, "FULL_PRECISION_FP16_COPY");
+    if (fsadam_clear_cache() != FSADAM_OK) bad |= 1;
+    printf(bad ? "FAILED\n" : "all modes bit-identical to the oracle\n");
+    return bad;
+}

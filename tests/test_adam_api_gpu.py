@@ -498,3 +498,29 @@ def test_walk_cost_for_four_thousand_tensors(api, cuda_device):
     assert opt.state[params[-1]]["step"] == 22
     print(f"steady-state host time per step, 4096 tensors: {steady * 1e3:.3f} ms")
     assert steady < 0.02  # generous: the Python walk took about 2 ms, the helper about 0.3 ms
+
+
+def test_added_param_group_steps_with_its_own_hyperparameters(api, cuda_device):
+    """``add_param_group`` after construction (the constructor itself takes a flat list, adam.py:90-91):
+    each group is one native call with its own lr / betas / weight decay, so two groups in one optimizer
+    give the same bits as two optimizers."""
+    Adam, _, _ = api
+    a = _random_problem("FULL_PRECISION", cuda_device, sizes=(100, 5000), seed=7)
+    b = _random_problem("FULL_PRECISION", cuda_device, sizes=(33, 140000), seed=8)
+    a2 = [p.detach().clone().requires_grad_() for p in a]
+    b2 = [p.detach().clone().requires_grad_() for p in b]
+    both = Adam(a, lr=1e-2)
+    both.add_param_group({"params": b, "lr": 3e-3, "betas": (0.8, 0.99), "weight_decay": 0.1})
+    one, two = Adam(a2, lr=1e-2), Adam(b2, lr=3e-3, betas=(0.8, 0.99), weight_decay=0.1)
+    for step in range(1, 5):
+        _set_grads(a, step, seed=7)
+        _set_grads(b, step, seed=8)
+        for src, dst in ((a, a2), (b, b2)):
+            for p, q in zip(src, dst):
+                q.grad = p.grad.clone()
+        both.step()
+        one.step()
+        two.step()
+    assert len(both._plans) == 2
+    for p, q in zip(a + b, a2 + b2):
+        assert torch.equal(p, q)
