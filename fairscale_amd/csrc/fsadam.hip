@@ -62,7 +62,7 @@ struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points a
     const void* g;
     void* p_copy;
     uint32_t n;          // elements in this chunk (<= chunk size of its launch)
-    uint32_t vector_ok;  // every stream aligned for the vector path
+    uint32_t vector_ok;  // full tiles of this chunk take the vector path
     uint64_t pad;
 };
 static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");
@@ -126,17 +126,23 @@ constexpr bool mode_has_copy(int mode) { return mode == FSADAM_MIXED_PRECISION |
 template <typename T, int E>
 struct VecOf {
     typedef T type __attribute__((ext_vector_type(E)));
+    // The same vector as it lies in memory: promised to be aligned like one element only.  Global
+    // memory instructions of this target take any address (code for amdhsa is generated under that
+    // assumption throughout), so the access is still one dwordx2/dwordx4 instruction; a stream
+    // that starts at an odd element (a view into a flat buffer) costs a cache line more per wave,
+    // not an element-by-element loop.
+    typedef type in_memory __attribute__((aligned(sizeof(T))));
 };
 
 // E consecutive elements of one stream, one instruction, non-temporal.
 template <typename T, int E>
 __device__ __forceinline__ typename VecOf<T, E>::type load_vec(gptr<const T> ptr) {
-    using V = typename VecOf<T, E>::type;
+    using V = typename VecOf<T, E>::in_memory;
     return __builtin_nontemporal_load(reinterpret_cast<gptr<const V>>(ptr));
 }
 template <typename T, int E>
 __device__ __forceinline__ void store_vec(gptr<T> ptr, typename VecOf<T, E>::type value) {
-    using V = typename VecOf<T, E>::type;
+    using V = typename VecOf<T, E>::in_memory;
     __builtin_nontemporal_store(value, reinterpret_cast<gptr<V>>(ptr));
 }
 
@@ -320,10 +326,18 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
 
 template <typename T>
 struct GradTraits;
+typedef uint32_t grad_words_t __attribute__((ext_vector_type(4)));
+// 16 bytes of gradients as they lie in memory: aligned like one element only (see VecOf::in_memory)
 template <>
-struct GradTraits<float> { static constexpr int kElems = 4; };
+struct GradTraits<float> {
+    static constexpr int kElems = 4;
+    typedef grad_words_t in_memory __attribute__((aligned(4)));
+};
 template <>
-struct GradTraits<_Float16> { static constexpr int kElems = 8; };
+struct GradTraits<_Float16> {
+    static constexpr int kElems = 8;
+    typedef grad_words_t in_memory __attribute__((aligned(2)));
+};
 
 // Magnitudes are compared as integers: with the sign bit cleared, IEEE bit patterns order like the
 // values, +inf is the largest finite-exponent pattern and every NaN is larger still.  One unsigned
@@ -404,13 +418,14 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, floa
     constexpr int E = GradTraits<T>::kElems;
     constexpr uint32_t kTile = BLOCK * E * ITEMS;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    using u32x4_in_memory = typename GradTraits<T>::in_memory;
     const uint32_t left = d.n - off;
     gptr<T> g = (gptr<T>)const_cast<void*>(d.g) + off;
     if (d.vector_ok && left >= kTile) {
         u32x4 raw[ITEMS];
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
-            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4>>(g + (k * BLOCK + threadIdx.x) * E));
+            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
         const f16x2 inv_half = {(_Float16)inv_scale, (_Float16)inv_scale};
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
@@ -423,7 +438,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, floa
                 else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
             }
             if (WRITE && HOW != kGradUnit)
-                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4>>(g + (k * BLOCK + threadIdx.x) * E));
+                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
         }
     } else {
         const uint32_t count = left < kTile ? left : kTile;
@@ -570,6 +585,7 @@ struct Options {
     int64_t grad_items = 0;     // gradient pass: 16-byte vectors per lane (2, 4 or 8; 0 = by kind of pass)
     int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
     int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
+    int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -846,7 +862,7 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     for (int64_t t = 0; t < n; ++t) {
         const FsAdamTensor& r = tensors[t];
         if (r.numel == 0) continue;
-        const bool vec = row_vector_ok(r, plan->mode);
+        const bool vec = plan->opt.unaligned_vectors != 0 || row_vector_ok(r, plan->mode);
         if (r.numel >= kLargeThreshold) {
             fill_descs(large, r, plan->mode, L.large_chunk_elems, vec);
             large += ceil_div(r.numel, L.large_chunk_elems);
@@ -909,6 +925,7 @@ struct GradPlan {
     int64_t items = 4;
     int64_t lds_throttle = 0;
     int64_t max_large_chunk = kMaxLargeChunk;
+    int64_t unaligned_vectors = 1;
     std::vector<FsGradTensor> rows;
     Layout layout;
     TableSlot slots[kTableSlots];
@@ -965,9 +982,10 @@ void grad_plan_free(GradPlan* plan) {
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
-void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk) {
+void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors) {
     std::lock_guard<std::mutex> lock(g_mutex);
     *max_large_chunk = g_opt.max_large_chunk;
+    *unaligned_vectors = g_opt.unaligned_vectors;
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
     *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 13312 : 16384);
 }
@@ -1024,7 +1042,7 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
             std::memset(&d, 0, sizeof(d));
             d.g = advance(r.g, c * chunk_elems, esz);
             d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - c * chunk_elems);
-            d.vector_ok = aligned_to(r.g, 16) ? 1u : 0u;
+            d.vector_ok = (plan->unaligned_vectors != 0 || aligned_to(r.g, 16)) ? 1u : 0u;
         }
         out += chunks;
     }
@@ -1107,7 +1125,7 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
 
 bool same_options(const Options& a, const Options& b) {
     return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap &&
-           a.max_large_chunk == b.max_large_chunk;
+           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors;
 }
 
 }  // namespace
@@ -1146,6 +1164,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "xcd_remap") {
         if (value < 0 || value > (1 << 28)) return fail(FSADAM_EINVAL, "xcd_remap must be 0 (off) or a run length in tiles");
         g_opt.xcd_remap = value;
+    } else if (k == "unaligned_vectors") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "unaligned_vectors must be 0 or 1");
+        g_opt.unaligned_vectors = value;
     } else if (k == "max_large_chunk") {
         if (value < 4096 || value > kMaxLargeChunk || (value & (value - 1)) != 0)
             return fail(FSADAM_EINVAL, "max_large_chunk must be a power of two in [4096, 2^24] elements");
@@ -1171,6 +1192,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "lds_throttle") *value = g_opt.lds_throttle;
     else if (k == "xcd_remap") *value = g_opt.xcd_remap;
     else if (k == "max_large_chunk") *value = g_opt.max_large_chunk;
+    else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
@@ -1317,14 +1339,14 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    int64_t cur_items, cur_lds, cur_chunk;
-    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk);
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned;
+    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            c->max_large_chunk == cur_chunk && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -1348,6 +1370,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->items = cur_items;
         victim->lds_throttle = cur_lds;
         victim->max_large_chunk = cur_chunk;
+        victim->unaligned_vectors = cur_unaligned;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;

@@ -72,8 +72,8 @@ typedef struct FsAdamPlanInfo {
     int64_t tile_elems;        /* elements one workgroup handles                                        */
     int64_t large_chunk_elems; /* elements per shared descriptor of a large tensor                      */
     int64_t n_descriptors;     /* 64-byte rows of the device table                                      */
-    int64_t n_vector_tensors;  /* tensors whose every stream is aligned for the 64/128-bit vector path  */
-    int64_t n_scalar_tensors;  /* tensors taking the element-wise path because of a misaligned stream   */
+    int64_t n_vector_tensors;  /* tensors whose every stream is aligned to its 64/128-bit vector         */
+    int64_t n_scalar_tensors;  /* tensors with a stream that is only element-aligned                    */
     int64_t n_launches;        /* kernel launches per step: 0 or 1                                      */
     int64_t grid;              /* workgroups per step, all launches                                     */
     int64_t block;             /* threads per workgroup                                                 */
@@ -118,6 +118,9 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
  *                   4 for one that writes the gradients back (default 0)
  *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
+ *   "unaligned_vectors"  1 (default): full tiles of a tensor whose streams are only element-aligned (a view that
+ *                   starts at an odd element) still move with 64/128-bit vector instructions; 0: such tensors
+ *                   are processed element by element (measured 1.5-2x slower)
  *   "max_large_chunk"    upper bound of the elements one shared descriptor of a large tensor covers: a
  *                   power of two in [4096, 2^24] (default 2^24; smaller values measured no faster)
  * Affects plans whose tensors are set after the call. */

@@ -4,6 +4,7 @@ transitions, error types), plus whole trajectories against the oracle's host sta
 from __future__ import annotations
 
 import copy
+import io
 
 import numpy as np
 import pytest
@@ -151,8 +152,14 @@ def test_state_dict_round_trip_keeps_lock_step(api, cuda_device, precision_name)
     w2 = w.data.clone().requires_grad_()
     b2 = b.data.clone().requires_grad_()
     opt2 = Adam([w2, b2], lr=1e-3, precision=precision)
-    sd = copy.deepcopy(opt.state_dict())
+    # through a file, with the loader that executes nothing: tensors, ints, floats and lists only
+    buffer = io.BytesIO()
+    torch.save(opt.state_dict(), buffer)
+    buffer.seek(0)
+    sd = torch.load(buffer, weights_only=True)
     assert sd["optim_scale"] == opt._optim_scale
+    assert set(sd) == {"state", "param_groups", "optim_scale"}
+    assert set(sd["state"][0]) == {"step", "exp_avg", "exp_avg_sq"}  # the reference's keys (adam.py:223-228)
     opt2.load_state_dict(sd)
     for p, q in ((w, w2), (b, b2)):
         for key in ("exp_avg", "exp_avg_sq"):

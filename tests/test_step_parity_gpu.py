@@ -131,12 +131,20 @@ def test_non_power_of_two_scales(oracle, cuda_device, mode):
 
 @pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
 @pytest.mark.parametrize("which", ["p", "g", "m", "all"])
-def test_misaligned_views(oracle, cuda_device, mode, which):
-    """Views that start 1 element (p: 3) into an allocation, like OSS bucket views: a stream that is
-    not aligned for the vector path sends the tensor down the element-wise path; results must not change."""
+@pytest.mark.parametrize("unaligned_vectors", [1, 0])
+def test_misaligned_views(oracle, cuda_device, mode, which, unaligned_vectors):
+    """Views that start 1 element (p: 3) into an allocation, like OSS bucket views.  By default their full
+    tiles still use vector instructions (at element-aligned addresses); with the option off the whole
+    tensor goes down the element-wise path.  Results must not change either way."""
+    from fairscale_amd import _cabi
+
     mis = {"p": {"p": 3}, "g": {"g": 1}, "m": {"m": 1}, "all": {"p": 1, "g": 1, "m": 1, "v": 1, "p16": 1}}[which]
-    run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000, 140001], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
-             grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
+    _cabi.set_option("unaligned_vectors", unaligned_vectors)
+    try:
+        run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000, 140001], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
+                 grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
+    finally:
+        _cabi.set_option("unaligned_vectors", 1)
 
 
 def test_steps_alternating_between_streams(oracle, cuda_device):
