@@ -167,6 +167,15 @@ __device__ __forceinline__ uint32_t nonfinite_in(typename VecOf<_Float16, E>::ty
     return bad;
 }
 
+// A float that is about to be narrowed to half passes through here first.  The compiler otherwise
+// merges "multiply, then convert" into one v_fma_mixlo_f16, which rounds the exact product once;
+// the reference (and the oracle) round to float32 first and to half afterwards, and the two differ
+// when the float32 result lands exactly between two halves.  No instruction is emitted.
+__device__ __forceinline__ float as_float32(float x) {
+    asm("" : "+v"(x));
+    return x;
+}
+
 // The update for one element, all in fp32 registers.
 //   unscaled state: fused_adam_cuda_kernel.cu:115-130     scaled (fp16) state: :94-114
 // out_m/out_v are what gets STORED (already multiplied by optim_scale when kScaled).
@@ -180,8 +189,8 @@ __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, fl
         const float v_un = FAST_SCALES ? in_v * s.inv_optim_scale : in_v / s.optim_scale;
         momentum = s.b1 * m_un + s.one_minus_b1 * scaled_grad;
         velocity = s.b2 * v_un + (s.one_minus_b2 * scaled_grad) * scaled_grad;
-        out_m = momentum * s.optim_scale;
-        out_v = velocity * s.optim_scale;
+        out_m = as_float32(momentum * s.optim_scale);
+        out_v = as_float32(velocity * s.optim_scale);
     } else {
         momentum = s.b1 * in_m + s.one_minus_b1 * scaled_grad;
         velocity = s.b2 * in_v + (s.one_minus_b2 * scaled_grad) * scaled_grad;
@@ -190,7 +199,7 @@ __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, fl
     }
     const float denom = (EPS_MODE == 0) ? sqrtf(velocity + s.eps) : sqrtf(velocity) + s.eps;
     const float update = momentum / denom + s.decay * in_p;
-    out_p = in_p - s.step_size * update;
+    out_p = as_float32(in_p - s.step_size * update);
 }
 
 // A full, aligned tile: GROUPS x (one vector per stream per lane), everything loaded before the
@@ -376,8 +385,8 @@ __device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2
     if (HOW == kGradHalfScale) {
         r = r * inv_half;
     } else if (HOW == kGradFloatScale) {
-        r[0] = (_Float16)((float)r[0] * inv_scale);
-        r[1] = (_Float16)((float)r[1] * inv_scale);
+        r[0] = (_Float16)as_float32((float)r[0] * inv_scale);
+        r[1] = (_Float16)as_float32((float)r[1] * inv_scale);
     }
     const uint32_t out = __builtin_bit_cast(uint32_t, r);
     if (HOW != kGradUnit) acc.stored_max = max_u16x2(acc.stored_max, out & 0x7fff7fffu);

@@ -62,6 +62,15 @@ def check(host, dev, stats, want, what):
         assert got_mx == mx, what
 
 
+def test_unscale_by_an_inexact_factor_rounds_twice_on_every_path(cuda_device):
+    """half(float32(float(g) * inv_scale)): the float32 rounding comes first, as in torch's kernel.  Many
+    tensors just below one tile (element-wise path) plus a large one (vector path), enough elements for
+    the one-in-10^4 cases where a single rounding of the exact product would differ."""
+    host = host_grads(np.float16, 31, [2047] * 300 + [500003], scale=3.0)
+    dev, stats, want = run_both(host, cuda_device, 1.0 / 3, True)
+    check(host, dev, stats, want, "inexact factor")
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("inv_scale", [1.0, 1.0 / 1024, 1.0 / 3])
 @pytest.mark.parametrize("write_back", [True, False])

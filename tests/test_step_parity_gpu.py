@@ -42,10 +42,11 @@ class GpuList:
 
     def _place(self, arrs, name):
         """Optionally put every tensor `k` elements into a larger allocation (a misaligned view)."""
-        k = self.misalign.get(name, 0)
+        shift = self.misalign.get(name, 0)
         out = []
-        for a in arrs:
+        for i, a in enumerate(arrs):
             t = torch.from_numpy(a).to(self.device)
+            k = shift[i] if isinstance(shift, (list, tuple)) else shift  # one offset for all, or one per tensor
             if k:
                 big = torch.empty(a.size + k + 8, dtype=t.dtype, device=self.device)
                 view = big[k:k + a.size]
@@ -173,6 +174,56 @@ def test_steps_alternating_between_streams(oracle, cuda_device):
         oracle_step(oracle, host, grads, flag, **kw)
         torch.cuda.synchronize(cuda_device)
         compare(host, dev, f"alternating streams, step {step}")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
+    """Differential test on drawn configurations: mode, list length, sizes around every boundary (empty,
+    below a tile, tile multiples +-1, around the large-tensor threshold), a separate element offset for
+    every stream of every tensor, eps placement, bias correction, decay, power-of-two or odd scales."""
+    import random
+
+    rng = random.Random(9000 + seed)
+    mode = rng.choice([FULL, MIXED, MEMEFF, PURE16])
+    tile = 512 if mode == PURE16 else 256
+
+    def draw_size():
+        kind = rng.randrange(6)
+        if kind == 0:
+            return rng.choice([0, 1, 2, 3])
+        if kind == 1:
+            return rng.randrange(4, tile)
+        if kind == 2:
+            return tile * rng.randrange(1, 40) + rng.choice([-1, 0, 1])
+        if kind == 3:
+            return rng.randrange(tile, 60000)
+        if kind == 4:
+            return 131072 + rng.choice([-1, 0, 1, 255, 257])
+        return rng.randrange(131072, 500000)
+
+    sizes = [draw_size() for _ in range(rng.randrange(1, 25))]
+    if sum(sizes) == 0:
+        sizes.append(77)
+    names = ["p", "m", "v", "g", "p16"]
+    misalign = {name: [rng.choice([0, 0, 1, 2, 3, 5, 7]) for _ in sizes] for name in names}
+    hyper = dict(lr=rng.choice([1e-3, 3e-2]), beta1=rng.choice([0.9, 0.5]), beta2=rng.choice([0.999, 0.95]),
+                 eps=rng.choice([1e-8, 1e-3]), eps_mode=rng.randrange(2), bias_correction=rng.randrange(2),
+                 decay=rng.choice([0.0, 0.01]))
+    grad_scale = rng.choice([1.0, 128.0, 3.0]) if mode != FULL else rng.choice([1.0, 3.0])
+    optim_scale = rng.choice([65536.0, 1024.0, 1000.0]) if mode == PURE16 else 1.0
+    print(f"seed {seed}: mode {mode}, {len(sizes)} tensors, {sum(sizes)} elements, grad_scale {grad_scale}, optim_scale {optim_scale}, {hyper}",
+          flush=True)
+    run_case(oracle, cuda_device, mode, sizes, 3, 9100 + seed, hyper, grad_scale=grad_scale, misalign=misalign,
+             optim_scale=optim_scale)
+
+
+def test_pure_fp16_odd_optim_scale_rounds_twice_on_every_path(oracle, cuda_device):
+    """m and v are stored as half(float32(m' * S)): two roundings (kernel.cu:100-101).  With a scale that is
+    not a power of two the float32 product is inexact, and about one element in 10^4 lands exactly between
+    two halves, where rounding the exact product once (a fused multiply-convert) gives the other
+    neighbour.  Tensors just below one tile run the element-wise path, the large one the vector path."""
+    run_case(oracle, cuda_device, PURE16, [511] * 300 + [300001], 3, 4700, dict(DEFAULT, lr=3e-2, beta1=0.5, eps=1e-3),
+             grad_scale=3.0, optim_scale=1000.0)
 
 
 def test_zero_sized_tensors_in_list(oracle, cuda_device):
