@@ -299,6 +299,62 @@ def test_trajectory_matches_oracle_state_machine(oracle, api, cuda_device, preci
     assert len(opt.state[params[0]]) == 0  # a parameter that never had a gradient keeps an empty state
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_trajectories_match_the_oracle_state_machine(oracle, api, cuda_device, seed):
+    """Drawn trajectories through the optimizer class: precision, list, hyper-parameters, a growth
+    interval of a few steps, gradients that go missing, a ``scale`` keyword, and (PURE_FP16) overflows
+    planted on drawn steps, so that backoff, zeroing and regrowth interleave.  Parameters, m, v, step
+    counters and the scale bookkeeping must follow ``OracleAdam`` bit for bit after every step."""
+    import random
+
+    Adam, _, Precision = api
+    rng = random.Random(6000 + seed)
+    precision_name = rng.choice(list(MODE_OF))
+    mode = MODE_OF[precision_name]
+    pd, gd, _ = C.MODE_DTYPES[mode]
+    host_dtype = np.float16 if mode != FULL else np.float32
+    sizes = [rng.choice([1, 5, 255, 256, 513, 4097, 20000, 131072, 200001]) for _ in range(rng.randrange(2, 9))]
+    nrng = np.random.default_rng(6100 + seed)
+    host = [(nrng.standard_normal(n).astype(np.float32) * 0.02).astype(host_dtype) for n in sizes]
+    hyper = dict(lr=rng.choice([1e-3, 1e-2]), betas=rng.choice([(0.9, 0.999), (0.8, 0.99)]), eps=rng.choice([1e-8, 1e-5]),
+                 weight_decay=rng.choice([0.0, 0.05]), bias_correction=rng.random() < 0.7, eps_inside_sqrt=rng.random() < 0.5)
+    scale = rng.choice([1.0, 64.0]) if mode != FULL else 1.0
+    params = [torch.from_numpy(h.copy()).to(cuda_device).requires_grad_() for h in host]
+    opt = Adam(params, precision=getattr(Precision, precision_name), **hyper)
+    ref = oracle.OracleAdam([h.copy() for h in host], mode, **hyper)
+    opt._optim_scale_update_freq = ref.optim_scale_update_freq = rng.choice([2, 3, 5])
+    overflow_steps = set(rng.sample(range(2, 13), 3)) if mode == PURE16 else set()
+    print(f"seed {seed}: {precision_name}, sizes {sizes}, {hyper}, scale {scale}, overflow on {sorted(overflow_steps)}", flush=True)
+    for step in range(1, 13):
+        grads = []
+        for j, n in enumerate(sizes):
+            if step > 1 and rng.random() < 0.1:
+                grads.append(None)
+                continue
+            g = (nrng.standard_normal(n).astype(np.float32) * np.float32(1e-3 * scale)).astype(gd)
+            if step in overflow_steps and j == len(sizes) - 1:
+                g[rng.randrange(n)] = np.float16(6e4)
+            grads.append(g)
+        if all(g is None for g in grads):
+            grads[0] = (nrng.standard_normal(sizes[0]).astype(np.float32) * np.float32(1e-3 * scale)).astype(gd)
+        for p, g in zip(params, grads):
+            p.grad = None if g is None else torch.from_numpy(g).to(cuda_device)
+        opt.step(scale=scale)
+        ref.step(grads, scale=scale)
+        assert opt._optim_scale == ref.optim_scale, f"step {step}"
+        assert opt._steps_since_optim_scale_change == ref.steps_since_optim_scale_change, f"step {step}"
+        for j, p in enumerate(params):
+            assert np.array_equal(p.detach().cpu().numpy().view(np.uint8), ref.params[j].view(np.uint8)), f"step {step} param {j}"
+            if ref.state[j].get("step") is not None:
+                st = opt.state[p]
+                assert st["step"] == ref.state[j]["step"], f"step {step} counter {j}"
+                for key in ("exp_avg", "exp_avg_sq"):
+                    assert np.array_equal(st[key].cpu().numpy().view(np.uint8), ref.state[j][key].view(np.uint8)), f"step {step} {key}[{j}]"
+        if mode == MIXED:
+            for j, master in enumerate(opt.fp32_param_groups[0]["params"]):
+                assert np.array_equal(master.detach().cpu().numpy(), ref.fp32_params[j]), f"step {step} master {j}"
+
+
 def test_scale_keyword_divides_the_gradients(oracle, api, cuda_device):
     """step(scale=s) on gradients multiplied by s gives the bits of step() on the plain gradients."""
     Adam, _, Precision = api

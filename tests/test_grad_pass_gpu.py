@@ -62,6 +62,57 @@ def check(host, dev, stats, want, what):
         assert got_mx == mx, what
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_gradient_lists_match_the_oracle(cuda_device, seed):
+    """Drawn configurations: dtype, list, sizes around the tile sizes of both kinds of pass, an element
+    offset per tensor, factors that are 1, a power of two, a half, not a half, tiny and huge, with and
+    without write-back, the factor on the host or on the device, special values planted."""
+    import random
+
+    rng = random.Random(7000 + seed)
+    dtype = rng.choice([np.float16, np.float32])
+
+    def draw_size():
+        kind = rng.randrange(5)
+        if kind == 0:
+            return rng.choice([0, 1, 2, 3, 7, 9])
+        if kind == 1:
+            return rng.choice([1024, 2048, 4096]) * rng.randrange(1, 6) + rng.choice([-1, 0, 1])
+        if kind == 2:
+            return rng.randrange(10, 5000)
+        if kind == 3:
+            return 131072 + rng.choice([-1, 0, 1])
+        return rng.randrange(131072, 400000)
+
+    sizes = [draw_size() for _ in range(rng.randrange(1, 20))]
+    if sum(sizes) == 0:
+        sizes.append(33)
+    inv_scale = rng.choice([1.0, 2.0 ** -7, 0.75, 1.0 / 3, 1e-4, 3e4 if dtype == np.float16 else 1e35])
+    write_back = rng.random() < 0.6
+    host = host_grads(dtype, 7100 + seed, sizes, scale=rng.choice([1.0, 1000.0]))
+    info = np.finfo(dtype)
+    if seed % 2:
+        for g in host:
+            for value in (np.inf, -np.inf, np.nan, info.max, -info.max, info.tiny, info.smallest_subnormal, 0.0, -0.0):
+                if g.size and rng.random() < 0.2:
+                    g[rng.randrange(g.size)] = value
+    print(f"seed {seed}: {np.dtype(dtype)}, {len(sizes)} tensors, {sum(sizes)} elements, inv_scale {inv_scale}, write_back {write_back}", flush=True)
+    from fairscale_amd.grad_pass import grad_pass
+
+    dev = []
+    for h in host:
+        k = rng.choice([0, 0, 1, 3, 5])
+        big = torch.empty(h.size + k + 8, dtype=torch.from_numpy(h).dtype, device=cuda_device)
+        view = big[k:k + h.size]
+        view.copy_(torch.from_numpy(h))
+        dev.append(view)
+    inv = torch.tensor([inv_scale], dtype=torch.float32, device=cuda_device) if rng.random() < 0.5 else inv_scale
+    stats = grad_pass(dev, inv, write_back=write_back)
+    torch.cuda.synchronize()
+    want = G.grad_pass_numpy(host, inv_scale, write_back)
+    check(host, dev, stats, want, f"seed {seed}")
+
+
 def test_unscale_by_an_inexact_factor_rounds_twice_on_every_path(cuda_device):
     """half(float32(float(g) * inv_scale)): the float32 rounding comes first, as in torch's kernel.  Many
     tensors just below one tile (element-wise path) plus a large one (vector path), enough elements for

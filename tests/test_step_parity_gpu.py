@@ -87,12 +87,15 @@ def compare(host: C.Tensors, dev: GpuList, tag: str, exact: bool = True):
     return inexact
 
 
-def run_case(oracle, device, mode, sizes, steps, seed, hyper, grad_scale=1.0, g_std=1e-3, misalign=None, optim_scale=1.0):
+def run_case(oracle, device, mode, sizes, steps, seed, hyper, grad_scale=1.0, g_std=1e-3, misalign=None, optim_scale=1.0,
+             mutate=None):
     host = C.Tensors(mode, sizes, seed)
     dev = GpuList(host, device, misalign)
     flag = np.zeros(1, np.float32)
     for step in range(1, steps + 1):
         grads = host.grads(step, g_std=g_std, scale=grad_scale)
+        if mutate is not None:
+            mutate(grads, step)
         kw = dict(hyper, step=step, grad_scale=grad_scale, optim_scale=optim_scale)
         dev.step(grads, **kw)
         oracle_step(oracle, host, grads, flag, **kw)
@@ -176,11 +179,13 @@ def test_steps_alternating_between_streams(oracle, cuda_device):
         compare(host, dev, f"alternating streams, step {step}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
     """Differential test on drawn configurations: mode, list length, sizes around every boundary (empty,
     below a tile, tile multiples +-1, around the large-tensor threshold), a separate element offset for
-    every stream of every tensor, eps placement, bias correction, decay, power-of-two or odd scales."""
+    every stream of every tensor, eps placement, bias correction, decay, power-of-two or odd scales;
+    every second seed also plants infinities, NaNs, the largest and the smallest magnitudes and zeros
+    in the gradients of the second step."""
     import random
 
     rng = random.Random(9000 + seed)
@@ -213,8 +218,19 @@ def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
     optim_scale = rng.choice([65536.0, 1024.0, 1000.0]) if mode == PURE16 else 1.0
     print(f"seed {seed}: mode {mode}, {len(sizes)} tensors, {sum(sizes)} elements, grad_scale {grad_scale}, optim_scale {optim_scale}, {hyper}",
           flush=True)
+    def plant(grads, step):
+        if step != 2 or seed % 2 == 0:
+            return
+        for g in grads:
+            if g.size == 0:
+                continue
+            info = np.finfo(g.dtype)
+            for value in (np.inf, -np.inf, np.nan, info.max, -info.max, info.tiny, info.smallest_subnormal, -info.smallest_subnormal, 0.0, -0.0):
+                if rng.random() < 0.3:
+                    g[rng.randrange(g.size)] = value
+
     run_case(oracle, cuda_device, mode, sizes, 3, 9100 + seed, hyper, grad_scale=grad_scale, misalign=misalign,
-             optim_scale=optim_scale)
+             optim_scale=optim_scale, mutate=plant)
 
 
 def test_pure_fp16_odd_optim_scale_rounds_twice_on_every_path(oracle, cuda_device):
