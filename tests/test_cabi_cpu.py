@@ -130,6 +130,43 @@ def test_layout_classes_and_descriptor_counts():
             _cabi.set_option(k, v)
 
 
+def test_layout_matches_a_python_model_on_drawn_lists():
+    """Descriptor and workgroup counts for drawn lists, modes and options against ten lines of Python."""
+    import random
+
+    rng = random.Random(42)
+    A = 0x7000_0000_0000
+    names = ("block", "groups", "max_large_chunk")
+    old = {k: _cabi.get_option(k) for k in names}
+    try:
+        for _ in range(60):
+            block, groups = rng.choice([64, 128, 256]), rng.choice([1, 2])
+            cap = rng.choice([1 << 24, 1 << 16, 1 << 14, 4096])
+            for k, v in zip(names, (block, groups, cap)):
+                _cabi.set_option(k, v)
+            mode = rng.choice([_cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16])
+            sizes = [rng.choice([0, 1, rng.randrange(2, 5000), rng.randrange(5000, 131072), 131072, rng.randrange(131072, 1 << 22),
+                                 rng.randrange(1 << 22, 1 << 31)]) for _ in range(rng.randrange(1, 30))]
+            tile = block * (8 if mode == _cabi.PURE_FP16 else 4) * groups
+            large = [n for n in sizes if n >= 131072]
+            chunk = 65536
+            if large:
+                chunk = 1 << ((min(large) // 2).bit_length() - 1)
+            chunk = min(cap, max(65536, min(1 << 24, chunk)))
+            want_large = sum(-(-n // chunk) for n in large)
+            want_small = sum(-(-n // tile) for n in sizes if 0 < n < 131072)
+            rows_ = [(A, A + (1 << 40), A + (2 << 40), A + (3 << 40), A + (4 << 40) if mode == _cabi.MIXED_PRECISION else 0, n) for n in sizes]
+            lay, cls, _ = layout(rows_, mode)
+            what = f"block {block} groups {groups} cap {cap} mode {mode} sizes {sizes}"
+            assert lay["tile_elems"] == tile and lay["large_chunk_elems"] == chunk, what
+            assert lay["n_large_descriptors"] == want_large and lay["n_small_descriptors"] == want_small, what
+            assert lay["grid_large"] == want_large * (chunk // tile) and lay["grid_small"] == want_small, what
+            assert cls == [0 if n == 0 else (2 if n >= 131072 else 1) for n in sizes], what
+    finally:
+        for k, v in old.items():
+            _cabi.set_option(k, v)
+
+
 def test_layout_alignment_rule_per_mode():
     A = 0x7000_0000_0000
     n = 1000
