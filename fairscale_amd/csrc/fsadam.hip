@@ -24,8 +24,9 @@
 // tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles; small tensors get
 // one descriptor per tile, placed after the large ones, so ONE launch covers any number of tensors
 // (the reference needs a launch per 36 tensors / 320 chunks because its table travels by value in
-// the kernel arguments).  Tiles that are ragged (end of a tensor) or belong to a tensor with a
-// misaligned stream take an element-wise path with the same arithmetic.
+// the kernel arguments).  Ragged tiles (the end of a tensor) take an element-wise path with the same
+// arithmetic; full tiles of a tensor whose streams are only element-aligned use the same vector
+// instructions at odd addresses.
 //
 // Arithmetic is IEEE float32 exactly as written in the reference source: separate multiplies and
 // adds (compiled with -ffp-contract=off), correctly rounded division and square root (hipcc's
@@ -202,7 +203,7 @@ __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, fl
     out_p = as_float32(in_p - s.step_size * update);
 }
 
-// A full, aligned tile: GROUPS x (one vector per stream per lane), everything loaded before the
+// A full tile: GROUPS x (one vector per stream per lane), everything loaded before the
 // first use.  Group k of the tile covers BLOCK*E consecutive elements, lane i the E elements at
 // k*BLOCK*E + i*E, so each instruction of a wave touches one contiguous span.
 template <int MODE, int BLOCK, int GROUPS, int EPS_MODE, bool FAST_SCALES>
@@ -251,7 +252,8 @@ __device__ __forceinline__ uint32_t tile_vector(const ChunkDesc& d, uint32_t off
     return bad;
 }
 
-// Ragged or misaligned tile: one element per lane per pass, same arithmetic.
+// Ragged tile (or, with the option unaligned_vectors off, a misaligned one): one element per lane per pass,
+// same arithmetic.
 template <int MODE, int BLOCK, int EPS_MODE, bool FAST_SCALES>
 __device__ __forceinline__ uint32_t tile_elementwise(const ChunkDesc& d, uint32_t off, uint32_t count, const StepScalars& s) {
     using T = ModeTraits<MODE>;
@@ -651,7 +653,7 @@ int validate_rows(const FsAdamTensor* tensors, int64_t n, int mode) {
     return FSADAM_OK;
 }
 
-// The vector path moves kElems elements per lane per instruction: each stream must be aligned to that.
+// Every stream aligned to the kElems elements a lane moves per instruction: the tensor runs at full speed.
 bool row_vector_ok(const FsAdamTensor& r, int mode) {
     const uintptr_t e = mode_elems(mode);
     return aligned_to(r.p, e * size_p(mode)) && aligned_to(r.m, e * size_s(mode)) && aligned_to(r.v, e * size_s(mode)) &&

@@ -163,7 +163,7 @@ int fsadam_plan_destroy(FsAdamPlan* plan);
 
 /* Host-only planning (no device needed): how the list would be laid out under the current options.
  * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large.  vector_ok[n_tensors] (may be
- * NULL): 1 = every stream aligned for the vector path. */
+ * NULL): 1 = every stream aligned to its 64/128-bit vector. */
 int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
                   uint8_t* tensor_class, uint8_t* vector_ok);
 
