@@ -1,4 +1,4 @@
-"""Compiles fsadam.hip into libfsadam.so next to this file (hipcc, gfx950 only), and the host-side
+"""Compiles fsadam.hip (with the kernel headers next to it) into libfsadam.so next to this file (hipcc, gfx950 only), and the host-side
 helper tensor_rows.cpp into a CPython extension module (g++, against the installed torch).
 
 Usage: ``python -m fairscale_amd.csrc.build``, or ``build_library()`` / ``build_rows_module()``.  Both
@@ -35,7 +35,7 @@ def hipcc_path() -> str:
 
 def build_library(verbose: bool = False) -> str:
     """Always recompiles; returns the path of the shared library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", INCLUDE, "-o", LIBRARY + ".tmp", SOURCE]
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", INCLUDE, "-I", HERE, "-o", LIBRARY + ".tmp", SOURCE]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"  # the host pass does not know the device feature
     log = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)

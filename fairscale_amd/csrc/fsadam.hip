@@ -1,4 +1,5 @@
-// Fused multi-tensor Adam step for MI355X (gfx950): kernels + C ABI (include/fsadam.h).
+// Fused multi-tensor Adam step for MI355X (gfx950): host code and C ABI (include/fsadam.h); the kernels
+// are in adam_kernels.h and grad_kernels.h, what both sides share in fsadam_common.h.
 //
 // Takes the place of fairscale's one native module:
 //   fairscale/clib/fused_adam_cuda/fused_adam_cuda_kernel.cu   (update equations :94-130, step size :153-162,
@@ -46,528 +47,11 @@
 
 #include "fsadam.h"
 
+#include "fsadam_common.h"
+#include "adam_kernels.h"
+#include "grad_kernels.h"
+
 namespace {
-
-// --------------------------------------------------------------------------------------------
-// shared host/device definitions
-// --------------------------------------------------------------------------------------------
-
-constexpr int64_t kLargeThreshold = 131072;   // tensors with at least this many elements share descriptors
-constexpr int64_t kMinLargeChunk = 65536;     // elements per shared descriptor, lower bound
-constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room); option max_large_chunk lowers it
-
-struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points at the chunk's first element
-    void* p;
-    void* m;
-    void* v;
-    const void* g;
-    void* p_copy;
-    uint32_t n;          // elements in this chunk (<= chunk size of its launch)
-    uint32_t vector_ok;  // full tiles of this chunk take the vector path
-    uint64_t pad;
-};
-static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");
-
-struct StepScalars {
-    float b1, b2, one_minus_b1, one_minus_b2;
-    float eps, decay, step_size;
-    float grad_scale, inv_grad_scale;
-    float optim_scale, inv_optim_scale;
-    int eps_mode;     // 0: sqrt(v+eps), 1: sqrt(v)+eps
-    int fast_scales;  // every scale the mode divides by is a power of two with an exact reciprocal
-};
-
-// Pointers read out of the descriptor table would otherwise be generic (flat_* instructions, which
-// also tie up the LDS counter); these live in global memory, so say so.
-#define FS_GLOBAL __attribute__((address_space(1)))
-template <typename T>
-using gptr = FS_GLOBAL T*;
-
-template <int MODE>
-struct ModeTraits;
-template <>
-struct ModeTraits<FSADAM_FULL_PRECISION> {
-    using P = float; using G = float; using S = float;
-    static constexpr bool kCopy = false, kScaled = false;
-    static constexpr int kElems = 4;  // elements per lane per group: 16 bytes of the widest stream
-};
-template <>
-struct ModeTraits<FSADAM_MIXED_PRECISION> {
-    using P = float; using G = _Float16; using S = float;
-    static constexpr bool kCopy = true, kScaled = false;
-    static constexpr int kElems = 4;
-};
-template <>
-struct ModeTraits<FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION> {
-    using P = _Float16; using G = _Float16; using S = float;
-    static constexpr bool kCopy = false, kScaled = false;
-    static constexpr int kElems = 4;
-};
-template <>
-struct ModeTraits<FSADAM_PURE_FP16> {
-    using P = _Float16; using G = _Float16; using S = _Float16;
-    static constexpr bool kCopy = false, kScaled = true;
-    static constexpr int kElems = 8;
-};
-
-template <>
-struct ModeTraits<FSADAM_FULL_PRECISION_FP16_COPY> {
-    using P = float; using G = float; using S = float;
-    static constexpr bool kCopy = true, kScaled = false;
-    static constexpr int kElems = 4;
-};
-
-constexpr int mode_elems(int mode) { return mode == FSADAM_PURE_FP16 ? 8 : 4; }
-constexpr bool mode_has_copy(int mode) { return mode == FSADAM_MIXED_PRECISION || mode == FSADAM_FULL_PRECISION_FP16_COPY; }
-
-// --------------------------------------------------------------------------------------------
-// device code
-// --------------------------------------------------------------------------------------------
-
-template <typename T, int E>
-struct VecOf {
-    typedef T type __attribute__((ext_vector_type(E)));
-    // The same vector as it lies in memory: promised to be aligned like one element only.  Global
-    // memory instructions of this target take any address (code for amdhsa is generated under that
-    // assumption throughout), so the access is still one dwordx2/dwordx4 instruction; a stream
-    // that starts at an odd element (a view into a flat buffer) costs a cache line more per wave,
-    // not an element-by-element loop.
-    typedef type in_memory __attribute__((aligned(sizeof(T))));
-};
-
-// E consecutive elements of one stream, one instruction, non-temporal.
-template <typename T, int E>
-__device__ __forceinline__ typename VecOf<T, E>::type load_vec(gptr<const T> ptr) {
-    using V = typename VecOf<T, E>::in_memory;
-    return __builtin_nontemporal_load(reinterpret_cast<gptr<const V>>(ptr));
-}
-template <typename T, int E>
-__device__ __forceinline__ void store_vec(gptr<T> ptr, typename VecOf<T, E>::type value) {
-    using V = typename VecOf<T, E>::in_memory;
-    __builtin_nontemporal_store(value, reinterpret_cast<gptr<V>>(ptr));
-}
-
-// Two packed halves in one 32-bit word: non-zero when either is +-inf or NaN (exponent field all
-// ones).  Adding 0x0400 to an all-ones exponent field carries into the sign position; any smaller
-// field does not, and the low half cannot carry into the high one.  Whole words, three integer
-// operations per two halves.  (A per-element form, __builtin_bit_cast(uint16_t, h[e]) on the elements
-// of a half vector, silently tested element 0 eight times: this compiler's bit_cast of a vector
-// ELEMENT always reads element 0.  Bit-cast whole vectors, or copy the element to a scalar first.)
-__device__ __forceinline__ uint32_t nonfinite_halves(uint32_t w) {
-    return ((w & 0x7c007c00u) + 0x04000400u) & 0x80008000u;
-}
-
-template <int E>
-__device__ __forceinline__ uint32_t nonfinite_in(typename VecOf<_Float16, E>::type h) {
-    static_assert(E == 4 || E == 8, "whole 32-bit words only");
-    typedef uint32_t words_t __attribute__((ext_vector_type(E / 2)));
-    const words_t w = __builtin_bit_cast(words_t, h);
-    uint32_t bad = 0;
-#pragma unroll
-    for (int k = 0; k < E / 2; ++k) bad |= nonfinite_halves(w[k]);
-    return bad;
-}
-
-// A float that is about to be narrowed to half passes through here first.  The compiler otherwise
-// merges "multiply, then convert" into one v_fma_mixlo_f16, which rounds the exact product once;
-// the reference (and the oracle) round to float32 first and to half afterwards, and the two differ
-// when the float32 result lands exactly between two halves.  No instruction is emitted.
-__device__ __forceinline__ float as_float32(float x) {
-    asm("" : "+v"(x));
-    return x;
-}
-
-// The update for one element, all in fp32 registers.
-//   unscaled state: fused_adam_cuda_kernel.cu:115-130     scaled (fp16) state: :94-114
-// out_m/out_v are what gets STORED (already multiplied by optim_scale when kScaled).
-template <bool kScaled, int EPS_MODE, bool FAST_SCALES>
-__device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, float in_m, float in_v, float in_g,
-                                            float& out_p, float& out_m, float& out_v) {
-    const float scaled_grad = FAST_SCALES ? in_g * s.inv_grad_scale : in_g / s.grad_scale;
-    float momentum, velocity;
-    if (kScaled) {
-        const float m_un = FAST_SCALES ? in_m * s.inv_optim_scale : in_m / s.optim_scale;
-        const float v_un = FAST_SCALES ? in_v * s.inv_optim_scale : in_v / s.optim_scale;
-        momentum = s.b1 * m_un + s.one_minus_b1 * scaled_grad;
-        velocity = s.b2 * v_un + (s.one_minus_b2 * scaled_grad) * scaled_grad;
-        out_m = as_float32(momentum * s.optim_scale);
-        out_v = as_float32(velocity * s.optim_scale);
-    } else {
-        momentum = s.b1 * in_m + s.one_minus_b1 * scaled_grad;
-        velocity = s.b2 * in_v + (s.one_minus_b2 * scaled_grad) * scaled_grad;
-        out_m = momentum;
-        out_v = velocity;
-    }
-    const float denom = (EPS_MODE == 0) ? sqrtf(velocity + s.eps) : sqrtf(velocity) + s.eps;
-    const float update = momentum / denom + s.decay * in_p;
-    out_p = as_float32(in_p - s.step_size * update);
-}
-
-// A full tile: GROUPS x (one vector per stream per lane), everything loaded before the
-// first use.  Group k of the tile covers BLOCK*E consecutive elements, lane i the E elements at
-// k*BLOCK*E + i*E, so each instruction of a wave touches one contiguous span.
-template <int MODE, int BLOCK, int GROUPS, int EPS_MODE, bool FAST_SCALES>
-__device__ __forceinline__ uint32_t tile_vector(const ChunkDesc& d, uint32_t off, const StepScalars& s) {
-    using T = ModeTraits<MODE>;
-    using P = typename T::P; using G = typename T::G; using S = typename T::S;
-    constexpr int E = T::kElems;
-    const uint32_t first = off + threadIdx.x * E;
-    gptr<P> p = (gptr<P>)d.p + first;
-    gptr<S> m = (gptr<S>)d.m + first;
-    gptr<S> v = (gptr<S>)d.v + first;
-    gptr<const G> g = (gptr<const G>)d.g + first;
-
-    typename VecOf<P, E>::type rp[GROUPS];
-    typename VecOf<S, E>::type rm[GROUPS], rv[GROUPS];
-    typename VecOf<G, E>::type rg[GROUPS];
-#pragma unroll
-    for (int k = 0; k < GROUPS; ++k) {
-        rp[k] = load_vec<P, E>(p + k * BLOCK * E);
-        rm[k] = load_vec<S, E>(m + k * BLOCK * E);
-        rv[k] = load_vec<S, E>(v + k * BLOCK * E);
-        rg[k] = load_vec<G, E>(g + k * BLOCK * E);
-    }
-    uint32_t bad = 0;
-#pragma unroll
-    for (int k = 0; k < GROUPS; ++k) {
-        typename VecOf<P, E>::type op;
-        typename VecOf<S, E>::type om, ov;
-        typename VecOf<_Float16, E>::type oc;
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            float np, nm, nv;
-            adam_update<T::kScaled, EPS_MODE, FAST_SCALES>(s, (float)rp[k][e], (float)rm[k][e], (float)rv[k][e],
-                                                           (float)rg[k][e], np, nm, nv);
-            op[e] = (P)np;  // round to nearest even when P is half
-            om[e] = (S)nm;
-            ov[e] = (S)nv;
-            if constexpr (T::kCopy) oc[e] = (_Float16)np;  // half(stored fp32 p): kernel.cu:129
-        }
-        if constexpr (T::kScaled) bad |= nonfinite_in<E>(om) | nonfinite_in<E>(ov);
-        store_vec<S, E>(m + k * BLOCK * E, om);
-        store_vec<S, E>(v + k * BLOCK * E, ov);
-        store_vec<P, E>(p + k * BLOCK * E, op);
-        if constexpr (T::kCopy) store_vec<_Float16, E>((gptr<_Float16>)d.p_copy + first + k * BLOCK * E, oc);
-    }
-    return bad;
-}
-
-// Ragged tile (or, with the option unaligned_vectors off, a misaligned one): one element per lane per pass,
-// same arithmetic.
-template <int MODE, int BLOCK, int EPS_MODE, bool FAST_SCALES>
-__device__ __forceinline__ uint32_t tile_elementwise(const ChunkDesc& d, uint32_t off, uint32_t count, const StepScalars& s) {
-    using T = ModeTraits<MODE>;
-    using P = typename T::P; using G = typename T::G; using S = typename T::S;
-    gptr<P> p = (gptr<P>)d.p + off;
-    gptr<S> m = (gptr<S>)d.m + off;
-    gptr<S> v = (gptr<S>)d.v + off;
-    gptr<const G> g = (gptr<const G>)d.g + off;
-    gptr<_Float16> pc = T::kCopy ? (gptr<_Float16>)d.p_copy + off : nullptr;
-    uint32_t bad = 0;
-    for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
-        float np, nm, nv;
-        adam_update<T::kScaled, EPS_MODE, FAST_SCALES>(s, (float)p[e], (float)m[e], (float)v[e], (float)g[e], np, nm, nv);
-        const S sm = (S)nm, sv = (S)nv;
-        m[e] = sm;
-        v[e] = sv;
-        if constexpr (T::kScaled)
-            bad |= nonfinite_halves((uint32_t)__builtin_bit_cast(uint16_t, sm) | ((uint32_t)__builtin_bit_cast(uint16_t, sv) << 16));
-        p[e] = (P)np;
-        if constexpr (T::kCopy) pc[e] = (_Float16)np;
-    }
-    return bad;
-}
-
-template <int MODE, int BLOCK, int GROUPS, int EPS_MODE, bool FAST_SCALES>
-__device__ __forceinline__ uint32_t tile_any(const ChunkDesc& d, uint32_t off, const StepScalars& s) {
-    constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
-    const uint32_t left = d.n - off;
-    if (d.vector_ok && left >= kTile) return tile_vector<MODE, BLOCK, GROUPS, EPS_MODE, FAST_SCALES>(d, off, s);
-    return tile_elementwise<MODE, BLOCK, EPS_MODE, FAST_SCALES>(d, off, left < kTile ? left : kTile, s);
-}
-
-// One workgroup = one tile.  The first `n_large_blocks` tiles belong to the descriptors of large
-// tensors, 2^log2k tiles each; every tile after them has a descriptor of its own (small tensors),
-// stored behind the `n_large_descs` large ones.  `n_blocks`: tiles really launched for (the grid may
-// be padded for the XCD remap).
-template <int MODE, int BLOCK, int GROUPS>
-__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
-                                                      uint32_t n_large_descs, uint32_t n_blocks, uint32_t xcd_stride,
-                                                      StepScalars s, float* __restrict__ found_inf) {
-    constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
-
-    uint32_t block = blockIdx.x;
-    if (xcd_stride) {
-        // Consecutive workgroups go to consecutive XCDs (eight L2s).  Regroup so that XCD x gets runs of
-        // `xcd_stride` consecutive tiles: within a group of 8*run workgroups, workgroup b takes tile
-        // (b % 8) * run + (b / 8) % run.
-        const uint32_t group = block / (8u * xcd_stride), in_group = block % (8u * xcd_stride);
-        block = group * 8u * xcd_stride + (in_group & 7u) * xcd_stride + (in_group >> 3);
-        if (block >= n_blocks) return;
-    }
-    const bool large = block < n_large_blocks;  // uniform: scalar selects
-    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
-    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
-    // The whole 64-byte descriptor in ONE scalar load (uniform address, constant address space), before
-    // anything is tested: reading the count first and the pointers afterwards would put two memory
-    // latencies in front of the first data load.
-    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
-    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
-        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
-    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
-    if (off >= d.n) return;  // tile past the end of its tensor (large tensors only)
-
-    uint32_t bad;
-    if (s.eps_mode == 0) {
-        bad = s.fast_scales ? tile_any<MODE, BLOCK, GROUPS, 0, true>(d, off, s) : tile_any<MODE, BLOCK, GROUPS, 0, false>(d, off, s);
-    } else {
-        bad = s.fast_scales ? tile_any<MODE, BLOCK, GROUPS, 1, true>(d, off, s) : tile_any<MODE, BLOCK, GROUPS, 1, false>(d, off, s);
-    }
-    // Same-value store from every lane that stored a non-finite fp16 m or v (kernel.cu:103-105).
-    if (ModeTraits<MODE>::kScaled && bad != 0) *(gptr<float>)found_inf = 1.0f;
-}
-
-
-// --------------------------------------------------------------------------------------------
-// gradient pass: non-finite check + unscale + sum of squares + max |g| in ONE read of the gradients
-// (what torch._amp_foreach_non_finite_check_and_unscale_, called from
-// fairscale/optim/grad_scaler.py:211-215, and calc_grad_norm, fairscale/internal/params.py:59-76,
-// do in two or more passes)
-// --------------------------------------------------------------------------------------------
-
-template <typename T>
-struct GradTraits;
-typedef uint32_t grad_words_t __attribute__((ext_vector_type(4)));
-// 16 bytes of gradients as they lie in memory: aligned like one element only (see VecOf::in_memory)
-template <>
-struct GradTraits<float> {
-    static constexpr int kElems = 4;
-    typedef grad_words_t in_memory __attribute__((aligned(4)));
-};
-template <>
-struct GradTraits<_Float16> {
-    static constexpr int kElems = 8;
-    typedef grad_words_t in_memory __attribute__((aligned(2)));
-};
-
-// Magnitudes are compared as integers: with the sign bit cleared, IEEE bit patterns order like the
-// values, +inf is the largest finite-exponent pattern and every NaN is larger still.  One unsigned
-// maximum therefore gives the max norm (a NaN wins, as in torch's abs().max()) and, taken over the
-// incoming values, the overflow check (maximum >= the pattern of +inf) -- no floating compare, no
-// per-element branch.  For halves two magnitudes travel in one 32-bit word (packed u16 maximum).
-struct GradPartial {  // one per workgroup, written unconditionally
-    double sum_squares;
-    uint32_t stored_max;    // largest magnitude pattern of the values unscaling stores
-    uint32_t incoming_max;  // largest magnitude pattern of the gradients as read
-};
-
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ uint32_t max_u16x2(uint32_t a, uint32_t b) {
-    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
-}
-
-// How the stored value r is formed from g: as is; by a packed half multiply (exact product, one
-// rounding: the same bits as float(g) * inv_scale rounded to half whenever inv_scale is itself a
-// half); or through float.
-enum : int { kGradUnit = 0, kGradHalfScale = 1, kGradFloatScale = 2 };
-
-struct GradAcc {
-    float sum = 0.f;
-    uint32_t stored_max = 0;
-    uint32_t incoming_max = 0;
-};
-
-// two halves in one word
-template <int HOW>
-__device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2 inv_half, GradAcc& acc) {
-    acc.incoming_max = max_u16x2(acc.incoming_max, w & 0x7fff7fffu);
-    f16x2 r = __builtin_bit_cast(f16x2, w);
-    if (HOW == kGradHalfScale) {
-        r = r * inv_half;
-    } else if (HOW == kGradFloatScale) {
-        r[0] = (_Float16)as_float32((float)r[0] * inv_scale);
-        r[1] = (_Float16)as_float32((float)r[1] * inv_scale);
-    }
-    const uint32_t out = __builtin_bit_cast(uint32_t, r);
-    if (HOW != kGradUnit) acc.stored_max = max_u16x2(acc.stored_max, out & 0x7fff7fffu);
-    // fused multiply-adds with half operands widened on the fly (v_fma_mix_f32): the product of two
-    // halves is exact in fp32, subnormal halves included
-    acc.sum = __builtin_fmaf((float)r[0], (float)r[0], acc.sum);
-    acc.sum = __builtin_fmaf((float)r[1], (float)r[1], acc.sum);
-    return out;
-}
-
-__device__ __forceinline__ _Float16 grad_scalar(_Float16 g, int how, float inv_scale, GradAcc& acc) {
-    const uint32_t w = __builtin_bit_cast(uint16_t, g);
-    uint32_t out;
-    if (how == kGradUnit) out = grad_word<kGradUnit>(w, inv_scale, f16x2{}, acc);
-    else out = grad_word<kGradFloatScale>(w, inv_scale, f16x2{}, acc);  // the two scaled forms give the same bits
-    return __builtin_bit_cast(_Float16, (uint16_t)out);
-}
-
-template <int HOW>
-__device__ __forceinline__ float grad_float(float g, float inv_scale, GradAcc& acc) {
-    const uint32_t mag = __builtin_bit_cast(uint32_t, g) & 0x7fffffffu;
-    acc.incoming_max = mag > acc.incoming_max ? mag : acc.incoming_max;
-    const float r = (HOW == kGradUnit) ? g : g * inv_scale;
-    if (HOW != kGradUnit) {
-        const uint32_t rm = __builtin_bit_cast(uint32_t, r) & 0x7fffffffu;
-        acc.stored_max = rm > acc.stored_max ? rm : acc.stored_max;
-    }
-    acc.sum += r * r;
-    return r;
-}
-
-__device__ __forceinline__ float grad_scalar(float g, int how, float inv_scale, GradAcc& acc) {
-    return how == kGradUnit ? grad_float<kGradUnit>(g, inv_scale, acc) : grad_float<kGradFloatScale>(g, inv_scale, acc);
-}
-
-template <typename T, int BLOCK, int ITEMS, int HOW, bool WRITE>
-__device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, float inv_scale, GradAcc& acc) {
-    constexpr int E = GradTraits<T>::kElems;
-    constexpr uint32_t kTile = BLOCK * E * ITEMS;
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    using u32x4_in_memory = typename GradTraits<T>::in_memory;
-    const uint32_t left = d.n - off;
-    gptr<T> g = (gptr<T>)const_cast<void*>(d.g) + off;
-    if (d.vector_ok && left >= kTile) {
-        u32x4 raw[ITEMS];
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k)
-            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
-        const f16x2 inv_half = {(_Float16)inv_scale, (_Float16)inv_scale};
-#pragma unroll
-        for (int k = 0; k < ITEMS; ++k) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // NB: copy the element out before __builtin_bit_cast: applied directly to a vector
-                // element (bit_cast(T, v[e])) this compiler reads element 0 whatever e is.
-                const uint32_t word = raw[k][e];
-                if constexpr (sizeof(T) == 2) raw[k][e] = grad_word<HOW>(word, inv_scale, inv_half, acc);
-                else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
-            }
-            if (WRITE && HOW != kGradUnit)
-                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
-        }
-    } else {
-        const uint32_t count = left < kTile ? left : kTile;
-        for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
-            const T r = grad_scalar(g[e], HOW, inv_scale, acc);
-            if (WRITE && HOW != kGradUnit) g[e] = r;
-        }
-    }
-}
-
-template <typename T, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
-                                                           uint32_t n_large_descs, float inv_scale_value,
-                                                           const float* __restrict__ inv_scale_dev, int write_back,
-                                                           GradPartial* __restrict__ partials) {
-    static_assert(BLOCK == 64, "one wave per workgroup: the partial is reduced with wave shuffles only");
-    constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
-    const uint32_t block = blockIdx.x;
-    const bool large = block < n_large_blocks;  // uniform: scalar selects
-    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
-    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
-    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
-    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
-        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
-    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
-    // the scale may live on the device (a loss scaler keeps it there): uniform address, scalar load
-    const float inv_scale = inv_scale_dev ? *(const __attribute__((address_space(4))) float*)inv_scale_dev : inv_scale_value;
-
-    GradAcc acc;
-    if (off < d.n) {
-        if (inv_scale == 1.0f) {
-            grad_tile<T, BLOCK, ITEMS, kGradUnit, false>(d, off, inv_scale, acc);
-        } else if (sizeof(T) == 2 && (float)(_Float16)inv_scale == inv_scale) {
-            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradHalfScale, true>(d, off, inv_scale, acc);
-            else grad_tile<T, BLOCK, ITEMS, kGradHalfScale, false>(d, off, inv_scale, acc);
-        } else {
-            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradFloatScale, true>(d, off, inv_scale, acc);
-            else grad_tile<T, BLOCK, ITEMS, kGradFloatScale, false>(d, off, inv_scale, acc);
-        }
-        if (inv_scale == 1.0f) acc.stored_max = acc.incoming_max;  // nothing was rescaled
-    }
-    if (sizeof(T) == 2) {  // unpack the two 16-bit maxima
-        acc.stored_max = (acc.stored_max & 0xffffu) > (acc.stored_max >> 16) ? (acc.stored_max & 0xffffu) : (acc.stored_max >> 16);
-        acc.incoming_max = (acc.incoming_max & 0xffffu) > (acc.incoming_max >> 16) ? (acc.incoming_max & 0xffffu) : (acc.incoming_max >> 16);
-    }
-    // wave reduction in a fixed order (xor butterfly): the same inputs always give the same bits
-    double dsum = (double)acc.sum;
-    uint32_t smax = acc.stored_max, imax = acc.incoming_max;
-#pragma unroll
-    for (int w = 32; w >= 1; w >>= 1) {
-        dsum += __shfl_xor(dsum, w, 64);
-        const uint32_t s2 = (uint32_t)__shfl_xor((int)smax, w, 64), i2 = (uint32_t)__shfl_xor((int)imax, w, 64);
-        smax = s2 > smax ? s2 : smax;
-        imax = i2 > imax ? i2 : imax;
-    }
-    if (threadIdx.x == 0) {
-        gptr<GradPartial> out = (gptr<GradPartial>)partials + block;
-        out->sum_squares = dsum;
-        out->stored_max = smax;
-        out->incoming_max = imax;
-    }
-}
-
-// Fixed-order reduction of `n` partials into `out[blockIdx.x]`: block b takes the b-th contiguous
-// slice, thread t every 256th entry of it, then a shared-memory tree.
-__global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
-                                                          GradPartial* __restrict__ out) {
-    __shared__ double s_sum[256];
-    __shared__ uint32_t s_stored[256];
-    __shared__ uint32_t s_incoming[256];
-    const uint32_t lo = blockIdx.x * per_block;
-    const uint32_t hi = lo + per_block < n ? lo + per_block : n;
-    double sum = 0.0;
-    uint32_t stored = 0, incoming = 0;
-    for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
-        const GradPartial p = in[i];
-        sum += p.sum_squares;
-        stored = p.stored_max > stored ? p.stored_max : stored;
-        incoming = p.incoming_max > incoming ? p.incoming_max : incoming;
-    }
-    s_sum[threadIdx.x] = sum; s_stored[threadIdx.x] = stored; s_incoming[threadIdx.x] = incoming;
-    __syncthreads();
-    for (int w = 128; w >= 1; w >>= 1) {
-        if ((int)threadIdx.x < w) {
-            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
-            s_stored[threadIdx.x] = s_stored[threadIdx.x + w] > s_stored[threadIdx.x] ? s_stored[threadIdx.x + w] : s_stored[threadIdx.x];
-            s_incoming[threadIdx.x] = s_incoming[threadIdx.x + w] > s_incoming[threadIdx.x] ? s_incoming[threadIdx.x + w] : s_incoming[threadIdx.x];
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        out[blockIdx.x].sum_squares = s_sum[0];
-        out[blockIdx.x].stored_max = s_stored[0];
-        out[blockIdx.x].incoming_max = s_incoming[0];
-    }
-}
-
-// Hands the single remaining partial to the caller's three outputs.
-__global__ void fsadam_grad_publish(const GradPartial* __restrict__ total, int is_half, float* found_inf, double* sum_squares,
-                                    float* abs_max) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
-        if (total->incoming_max >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
-        if (sum_squares) *sum_squares = total->sum_squares;
-        if (abs_max)
-            *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)total->stored_max) : __builtin_bit_cast(float, total->stored_max);
-    }
-}
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-template <int BLOCK>
-__global__ __launch_bounds__(BLOCK) void fsadam_copy_kernel(f32x4* __restrict__ dst_, const f32x4* __restrict__ src_, int64_t n_quads) {
-    gptr<f32x4> dst = (gptr<f32x4>)dst_;
-    gptr<const f32x4> src = (gptr<const f32x4>)src_;
-    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    if (i < n_quads) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
-}
 
 // --------------------------------------------------------------------------------------------
 // host side

@@ -1,0 +1,254 @@
+// Device code of the pre-step gradient pass (fsadam_grad_tiles, its two reduction kernels) and the
+// plain copy kernel used to calibrate the profiler's traffic counters.
+// Included by fsadam.hip only (one translation unit).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "fsadam_common.h"
+#include "adam_kernels.h"
+
+namespace {
+
+// --------------------------------------------------------------------------------------------
+// gradient pass: non-finite check + unscale + sum of squares + max |g| in ONE read of the gradients
+// (what torch._amp_foreach_non_finite_check_and_unscale_, called from
+// fairscale/optim/grad_scaler.py:211-215, and calc_grad_norm, fairscale/internal/params.py:59-76,
+// do in two or more passes)
+// --------------------------------------------------------------------------------------------
+
+template <typename T>
+struct GradTraits;
+typedef uint32_t grad_words_t __attribute__((ext_vector_type(4)));
+// 16 bytes of gradients as they lie in memory: aligned like one element only (see VecOf::in_memory)
+template <>
+struct GradTraits<float> {
+    static constexpr int kElems = 4;
+    typedef grad_words_t in_memory __attribute__((aligned(4)));
+};
+template <>
+struct GradTraits<_Float16> {
+    static constexpr int kElems = 8;
+    typedef grad_words_t in_memory __attribute__((aligned(2)));
+};
+
+// Magnitudes are compared as integers: with the sign bit cleared, IEEE bit patterns order like the
+// values, +inf is the largest finite-exponent pattern and every NaN is larger still.  One unsigned
+// maximum therefore gives the max norm (a NaN wins, as in torch's abs().max()) and, taken over the
+// incoming values, the overflow check (maximum >= the pattern of +inf) -- no floating compare, no
+// per-element branch.  For halves two magnitudes travel in one 32-bit word (packed u16 maximum).
+struct GradPartial {  // one per workgroup, written unconditionally
+    double sum_squares;
+    uint32_t stored_max;    // largest magnitude pattern of the values unscaling stores
+    uint32_t incoming_max;  // largest magnitude pattern of the gradients as read
+};
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t max_u16x2(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
+
+// How the stored value r is formed from g: as is; by a packed half multiply (exact product, one
+// rounding: the same bits as float(g) * inv_scale rounded to half whenever inv_scale is itself a
+// half); or through float.
+enum : int { kGradUnit = 0, kGradHalfScale = 1, kGradFloatScale = 2 };
+
+struct GradAcc {
+    float sum = 0.f;
+    uint32_t stored_max = 0;
+    uint32_t incoming_max = 0;
+};
+
+// two halves in one word
+template <int HOW>
+__device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2 inv_half, GradAcc& acc) {
+    acc.incoming_max = max_u16x2(acc.incoming_max, w & 0x7fff7fffu);
+    f16x2 r = __builtin_bit_cast(f16x2, w);
+    if (HOW == kGradHalfScale) {
+        r = r * inv_half;
+    } else if (HOW == kGradFloatScale) {
+        r[0] = (_Float16)as_float32((float)r[0] * inv_scale);
+        r[1] = (_Float16)as_float32((float)r[1] * inv_scale);
+    }
+    const uint32_t out = __builtin_bit_cast(uint32_t, r);
+    if (HOW != kGradUnit) acc.stored_max = max_u16x2(acc.stored_max, out & 0x7fff7fffu);
+    // fused multiply-adds with half operands widened on the fly (v_fma_mix_f32): the product of two
+    // halves is exact in fp32, subnormal halves included
+    acc.sum = __builtin_fmaf((float)r[0], (float)r[0], acc.sum);
+    acc.sum = __builtin_fmaf((float)r[1], (float)r[1], acc.sum);
+    return out;
+}
+
+__device__ __forceinline__ _Float16 grad_scalar(_Float16 g, int how, float inv_scale, GradAcc& acc) {
+    const uint32_t w = __builtin_bit_cast(uint16_t, g);
+    uint32_t out;
+    if (how == kGradUnit) out = grad_word<kGradUnit>(w, inv_scale, f16x2{}, acc);
+    else out = grad_word<kGradFloatScale>(w, inv_scale, f16x2{}, acc);  // the two scaled forms give the same bits
+    return __builtin_bit_cast(_Float16, (uint16_t)out);
+}
+
+template <int HOW>
+__device__ __forceinline__ float grad_float(float g, float inv_scale, GradAcc& acc) {
+    const uint32_t mag = __builtin_bit_cast(uint32_t, g) & 0x7fffffffu;
+    acc.incoming_max = mag > acc.incoming_max ? mag : acc.incoming_max;
+    const float r = (HOW == kGradUnit) ? g : g * inv_scale;
+    if (HOW != kGradUnit) {
+        const uint32_t rm = __builtin_bit_cast(uint32_t, r) & 0x7fffffffu;
+        acc.stored_max = rm > acc.stored_max ? rm : acc.stored_max;
+    }
+    acc.sum += r * r;
+    return r;
+}
+
+__device__ __forceinline__ float grad_scalar(float g, int how, float inv_scale, GradAcc& acc) {
+    return how == kGradUnit ? grad_float<kGradUnit>(g, inv_scale, acc) : grad_float<kGradFloatScale>(g, inv_scale, acc);
+}
+
+template <typename T, int BLOCK, int ITEMS, int HOW, bool WRITE>
+__device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, float inv_scale, GradAcc& acc) {
+    constexpr int E = GradTraits<T>::kElems;
+    constexpr uint32_t kTile = BLOCK * E * ITEMS;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    using u32x4_in_memory = typename GradTraits<T>::in_memory;
+    const uint32_t left = d.n - off;
+    gptr<T> g = (gptr<T>)const_cast<void*>(d.g) + off;
+    if (d.vector_ok && left >= kTile) {
+        u32x4 raw[ITEMS];
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k)
+            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
+        const f16x2 inv_half = {(_Float16)inv_scale, (_Float16)inv_scale};
+#pragma unroll
+        for (int k = 0; k < ITEMS; ++k) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // NB: copy the element out before __builtin_bit_cast: applied directly to a vector
+                // element (bit_cast(T, v[e])) this compiler reads element 0 whatever e is.
+                const uint32_t word = raw[k][e];
+                if constexpr (sizeof(T) == 2) raw[k][e] = grad_word<HOW>(word, inv_scale, inv_half, acc);
+                else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
+            }
+            if (WRITE && HOW != kGradUnit)
+                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
+        }
+    } else {
+        const uint32_t count = left < kTile ? left : kTile;
+        for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
+            const T r = grad_scalar(g[e], HOW, inv_scale, acc);
+            if (WRITE && HOW != kGradUnit) g[e] = r;
+        }
+    }
+}
+
+template <typename T, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
+                                                           uint32_t n_large_descs, float inv_scale_value,
+                                                           const float* __restrict__ inv_scale_dev, int write_back,
+                                                           GradPartial* __restrict__ partials) {
+    static_assert(BLOCK == 64, "one wave per workgroup: the partial is reduced with wave shuffles only");
+    constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
+    const uint32_t block = blockIdx.x;
+    const bool large = block < n_large_blocks;  // uniform: scalar selects
+    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
+    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
+    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
+    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
+        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
+    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    // the scale may live on the device (a loss scaler keeps it there): uniform address, scalar load
+    const float inv_scale = inv_scale_dev ? *(const __attribute__((address_space(4))) float*)inv_scale_dev : inv_scale_value;
+
+    GradAcc acc;
+    if (off < d.n) {
+        if (inv_scale == 1.0f) {
+            grad_tile<T, BLOCK, ITEMS, kGradUnit, false>(d, off, inv_scale, acc);
+        } else if (sizeof(T) == 2 && (float)(_Float16)inv_scale == inv_scale) {
+            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradHalfScale, true>(d, off, inv_scale, acc);
+            else grad_tile<T, BLOCK, ITEMS, kGradHalfScale, false>(d, off, inv_scale, acc);
+        } else {
+            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradFloatScale, true>(d, off, inv_scale, acc);
+            else grad_tile<T, BLOCK, ITEMS, kGradFloatScale, false>(d, off, inv_scale, acc);
+        }
+        if (inv_scale == 1.0f) acc.stored_max = acc.incoming_max;  // nothing was rescaled
+    }
+    if (sizeof(T) == 2) {  // unpack the two 16-bit maxima
+        acc.stored_max = (acc.stored_max & 0xffffu) > (acc.stored_max >> 16) ? (acc.stored_max & 0xffffu) : (acc.stored_max >> 16);
+        acc.incoming_max = (acc.incoming_max & 0xffffu) > (acc.incoming_max >> 16) ? (acc.incoming_max & 0xffffu) : (acc.incoming_max >> 16);
+    }
+    // wave reduction in a fixed order (xor butterfly): the same inputs always give the same bits
+    double dsum = (double)acc.sum;
+    uint32_t smax = acc.stored_max, imax = acc.incoming_max;
+#pragma unroll
+    for (int w = 32; w >= 1; w >>= 1) {
+        dsum += __shfl_xor(dsum, w, 64);
+        const uint32_t s2 = (uint32_t)__shfl_xor((int)smax, w, 64), i2 = (uint32_t)__shfl_xor((int)imax, w, 64);
+        smax = s2 > smax ? s2 : smax;
+        imax = i2 > imax ? i2 : imax;
+    }
+    if (threadIdx.x == 0) {
+        gptr<GradPartial> out = (gptr<GradPartial>)partials + block;
+        out->sum_squares = dsum;
+        out->stored_max = smax;
+        out->incoming_max = imax;
+    }
+}
+
+// Fixed-order reduction of `n` partials into `out[blockIdx.x]`: block b takes the b-th contiguous
+// slice, thread t every 256th entry of it, then a shared-memory tree.
+__global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
+                                                          GradPartial* __restrict__ out) {
+    __shared__ double s_sum[256];
+    __shared__ uint32_t s_stored[256];
+    __shared__ uint32_t s_incoming[256];
+    const uint32_t lo = blockIdx.x * per_block;
+    const uint32_t hi = lo + per_block < n ? lo + per_block : n;
+    double sum = 0.0;
+    uint32_t stored = 0, incoming = 0;
+    for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+        const GradPartial p = in[i];
+        sum += p.sum_squares;
+        stored = p.stored_max > stored ? p.stored_max : stored;
+        incoming = p.incoming_max > incoming ? p.incoming_max : incoming;
+    }
+    s_sum[threadIdx.x] = sum; s_stored[threadIdx.x] = stored; s_incoming[threadIdx.x] = incoming;
+    __syncthreads();
+    for (int w = 128; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+            s_stored[threadIdx.x] = s_stored[threadIdx.x + w] > s_stored[threadIdx.x] ? s_stored[threadIdx.x + w] : s_stored[threadIdx.x];
+            s_incoming[threadIdx.x] = s_incoming[threadIdx.x + w] > s_incoming[threadIdx.x] ? s_incoming[threadIdx.x + w] : s_incoming[threadIdx.x];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        out[blockIdx.x].sum_squares = s_sum[0];
+        out[blockIdx.x].stored_max = s_stored[0];
+        out[blockIdx.x].incoming_max = s_incoming[0];
+    }
+}
+
+// Hands the single remaining partial to the caller's three outputs.
+__global__ void fsadam_grad_publish(const GradPartial* __restrict__ total, int is_half, float* found_inf, double* sum_squares,
+                                    float* abs_max) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
+        if (total->incoming_max >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
+        if (sum_squares) *sum_squares = total->sum_squares;
+        if (abs_max)
+            *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)total->stored_max) : __builtin_bit_cast(float, total->stored_max);
+    }
+}
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fsadam_copy_kernel(f32x4* __restrict__ dst_, const f32x4* __restrict__ src_, int64_t n_quads) {
+    gptr<f32x4> dst = (gptr<f32x4>)dst_;
+    gptr<const f32x4> src = (gptr<const f32x4>)src_;
+    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i < n_quads) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+}  // namespace
