@@ -75,6 +75,8 @@ SIGNATURES = {
     "fsadam_plan_create": (_i32, [_i32, ctypes.POINTER(_vp)]),
     "fsadam_plan_set_tensors": (_i32, [_vp, ctypes.POINTER(FsAdamTensor), _i64, _vp]),
     "fsadam_plan_step": (_i32, [_vp] + _SCALARS + [_vp, _vp]),
+    # lr, beta1, beta2, eps, grad_scale_dev, optim_scale, decay, step, eps_mode, bias_correction, found_inf, stream
+    "fsadam_plan_step_dev_scale": (_i32, [_vp, _f32, _f32, _f32, _f32, _vp, _f32, _f32, _i32, _i32, _i32, _vp, _vp]),
     "fsadam_plan_info": (_i32, [_vp, ctypes.POINTER(FsAdamPlanInfo)]),
     "fsadam_plan_destroy": (_i32, [_vp]),
     "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),

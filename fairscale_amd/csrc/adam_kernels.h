@@ -205,6 +205,10 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
     const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
         (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
     const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    // A gradient scale that lives on the device (a clip factor or a loss scale computed there): one more
+    // scalar load at a uniform address, issued next to the descriptor's.  The host has already switched
+    // to true division (fast_scales = 0), which gives the bits of a host-side scale of the same value.
+    if (s.grad_scale_dev) s.grad_scale = *(const __attribute__((address_space(4))) float*)s.grad_scale_dev;
     if (off >= d.n) return;  // tile past the end of its tensor (large tensors only)
 
     uint32_t bad;

@@ -377,8 +377,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     return FSADAM_OK;
 }
 
-int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, float grad_scale, float optim_scale,
-              float decay, int step, int eps_mode, int bias_correction, float* found_inf, hipStream_t stream) {
+int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, float grad_scale, const float* grad_scale_dev,
+              float optim_scale, float decay, int step, int eps_mode, int bias_correction, float* found_inf, hipStream_t stream) {
     if (plan->rows.empty() || plan->current < 0) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
     if (eps_mode != FSADAM_EPS_INSIDE_SQRT && eps_mode != FSADAM_EPS_OUTSIDE_SQRT)
         return fail(FSADAM_EINVAL, "eps_mode must be 0 (inside sqrt) or 1 (outside)");
@@ -397,7 +397,8 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     s.grad_scale = grad_scale; s.optim_scale = optim_scale;
     s.inv_grad_scale = 0.f; s.inv_optim_scale = 0.f;
     s.eps_mode = eps_mode;
-    const bool gs_ok = is_pow2_with_exact_reciprocal(grad_scale, &s.inv_grad_scale);
+    s.grad_scale_dev = grad_scale_dev;
+    const bool gs_ok = grad_scale_dev == nullptr && is_pow2_with_exact_reciprocal(grad_scale, &s.inv_grad_scale);
     const bool os_ok = is_pow2_with_exact_reciprocal(optim_scale, &s.inv_optim_scale);
     s.fast_scales = (gs_ok && (plan->mode != FSADAM_PURE_FP16 || os_ok)) ? 1 : 0;
 
@@ -740,7 +741,17 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
                      float optim_scale, float decay, int step, int eps_mode, int bias_correction,
                      float* found_inf_dev, void* hip_stream) {
     if (!plan) return fail(FSADAM_EINVAL, "plan is NULL");
-    return plan_step(plan, lr, beta1, beta2, eps, grad_scale, optim_scale, decay, step, eps_mode, bias_correction,
+    return plan_step(plan, lr, beta1, beta2, eps, grad_scale, nullptr, optim_scale, decay, step, eps_mode, bias_correction,
+                     found_inf_dev, static_cast<hipStream_t>(hip_stream));
+}
+
+int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, const float* grad_scale_dev,
+                               float optim_scale, float decay, int step, int eps_mode, int bias_correction,
+                               float* found_inf_dev, void* hip_stream) {
+    if (!plan) return fail(FSADAM_EINVAL, "plan is NULL");
+    if (!grad_scale_dev) return fail(FSADAM_EINVAL, "grad_scale_dev is NULL");
+    if (!aligned_to(grad_scale_dev, 4)) return fail(FSADAM_EINVAL, "grad_scale_dev is not aligned to 4 bytes");
+    return plan_step(plan, lr, beta1, beta2, eps, 1.0f, grad_scale_dev, optim_scale, decay, step, eps_mode, bias_correction,
                      found_inf_dev, static_cast<hipStream_t>(hip_stream));
 }
 
@@ -815,7 +826,7 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
         hit = victim;
     }
     hit->lru = ++g_tick;
-    return plan_step(hit, lr, beta1, beta2, eps, grad_scale, optim_scale, decay, step, eps_mode, bias_correction,
+    return plan_step(hit, lr, beta1, beta2, eps, grad_scale, nullptr, optim_scale, decay, step, eps_mode, bias_correction,
                      found_inf_dev, stream);
 }
 

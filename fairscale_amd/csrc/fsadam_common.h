@@ -30,6 +30,7 @@ struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points a
 static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");
 
 struct StepScalars {
+    const float* grad_scale_dev;  // when not NULL the kernel reads the gradient scale here instead of grad_scale
     float b1, b2, one_minus_b1, one_minus_b2;
     float eps, decay, step_size;
     float grad_scale, inv_grad_scale;

@@ -211,17 +211,26 @@ class TensorListPlan:
     def step_rows(self, changed: bool, lr: float, beta1: float, beta2: float, eps: float, grad_scale: float,
                   optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int, bias_correction: int,
                   decay: float) -> None:
-        """Step over the rows already written into ``rows_buffer`` (validated by whoever wrote them)."""
+        """Step over the rows already written into ``rows_buffer`` (validated by whoever wrote them).
+        ``grad_scale`` is a Python float or a one-element float32 tensor on the plan's device, which the
+        kernel reads when it runs (no host synchronisation)."""
         L = _cabi.lib()
         rows = self._rows
+        scale_on_device = isinstance(grad_scale, torch.Tensor)
+        if scale_on_device and (grad_scale.dtype != torch.float32 or grad_scale.numel() != 1 or grad_scale.device != self.device):
+            raise RuntimeError("a tensor scale must be float32 with one element on the parameters' device")
         with torch.cuda.device(self.device):
             stream = _stream_handle(self.device)
             if changed or self._dirty:
                 _cabi.check(L.fsadam_plan_set_tensors(self._handle, _rows_ptr(rows), rows.shape[0], stream))
                 self._dirty = False
             flag = found_inf.data_ptr() if found_inf is not None else None
-            _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, grad_scale, optim_scale, decay,
-                                           int(step), int(eps_mode), int(bias_correction), flag, stream))
+            if scale_on_device:
+                _cabi.check(L.fsadam_plan_step_dev_scale(self._handle, lr, beta1, beta2, eps, grad_scale.data_ptr(), optim_scale,
+                                                         decay, int(step), int(eps_mode), int(bias_correction), flag, stream))
+            else:
+                _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, grad_scale, optim_scale, decay,
+                                               int(step), int(eps_mode), int(bias_correction), flag, stream))
 
     def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,
              grad_scale: float, optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int,

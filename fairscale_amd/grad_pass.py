@@ -130,14 +130,17 @@ def calc_grad_norm(parameters: Union[torch.Tensor, Iterable[torch.nn.Parameter]]
 
 
 def clip_grad_norm_(parameters: Union[torch.Tensor, Iterable[torch.nn.Parameter]], max_norm: Union[float, int],
-                    norm_type: Union[float, int] = 2.0, *, fold: bool = False) -> Union[torch.Tensor, Tuple[torch.Tensor, float]]:
+                    norm_type: Union[float, int] = 2.0, *,
+                    fold: Union[bool, str] = False) -> Union[torch.Tensor, Tuple[torch.Tensor, Union[float, torch.Tensor]]]:
     """One rank's part of ``OSS.clip_grad_norm`` (``oss.py:244-302``) / FSDP ``clip_grad_norm_``: the total
     norm, and gradients multiplied in place by ``max_norm / (norm + 1e-6)`` when that is below 1.
     (Across ranks the callers all-reduce ``norm**p`` in between; that stays with them.)
 
     ``fold=True`` skips the multiplication and returns ``(total_norm, grad_scale)`` instead, where
     ``grad_scale`` (>= 1) is the factor to hand to ``Adam.step(scale=...)``: the step then divides by it
-    in registers, which saves a read and a write of every gradient.
+    in registers, which saves a read and a write of every gradient.  ``fold="device"`` does the same
+    without the host read-back: ``grad_scale`` is then a one-element float32 tensor on the norm's
+    device holding the same value, which the step kernel reads when it runs.
     """
     if isinstance(parameters, torch.Tensor):
         parameters = [parameters]
@@ -147,6 +150,10 @@ def clip_grad_norm_(parameters: Union[torch.Tensor, Iterable[torch.nn.Parameter]
     if len(params) == 0:
         return (total_norm, 1.0) if fold else total_norm
     clip_coef = torch.tensor(max_norm, dtype=total_norm.dtype, device=total_norm.device) / (total_norm + 1e-6)
+    if fold == "device":
+        # 1 / clip_coef evaluated in float64 and narrowed, as float(1.0 / float(clip_coef)) is on the host
+        factor = clip_coef.double().reciprocal().float()
+        return total_norm, torch.where(clip_coef < 1, factor, torch.ones_like(factor)).reshape(1)
     clipping = bool(clip_coef < 1)  # the reference's host read-back (oss.py:297)
     if fold:
         return total_norm, (1.0 / float(clip_coef)) if clipping else 1.0

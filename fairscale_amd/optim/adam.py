@@ -23,7 +23,7 @@ from __future__ import annotations
 from collections import defaultdict
 from enum import Enum, auto
 from operator import is_not
-from typing import Any, Callable, Dict, List, Optional, Tuple
+from typing import Any, Callable, Dict, List, Optional, Tuple, Union
 
 import torch
 
@@ -364,12 +364,15 @@ class Adam(torch.optim.Optimizer):
             lists.append(outs)
         return {device: lists}, states[-1]["step"]
 
-    def step(self, closure: Optional[Callable[[], float]] = None, *, scale: float = 1.0) -> Optional[float]:
+    def step(self, closure: Optional[Callable[[], float]] = None, *, scale: Union[float, torch.Tensor] = 1.0) -> Optional[float]:
         """One optimization step (adam.py:184-297).
 
         Arguments:
             closure: re-evaluates the model and returns the loss.
-            scale: gradients are divided by this inside the kernel (loss-scale folded into the step).
+            scale: gradients are divided by this inside the kernel (loss scale or clip factor folded
+                into the step).  A Python float, or a one-element float32 tensor on the parameters'
+                device that the kernel reads when it runs, so that a factor computed on the device
+                (``clip_grad_norm_(..., fold="device")``) costs no host synchronisation.
         """
         loss = closure() if closure is not None else None
         self.__dict__.setdefault("_plans", {})  # absent after unpickling

@@ -161,6 +161,16 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
 int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out);
 int fsadam_plan_destroy(FsAdamPlan* plan);
 
+/* As fsadam_plan_step, with the gradient scale read by the kernel from device memory (one float that must be
+ * valid when the kernel runs; nothing is synchronised on the host).  For callers that compute the scale
+ * on the device: a clip factor max(1, norm / max_norm) from fsadam_grad_pass's sum of squares, or a loss
+ * scale kept in a device tensor.  The result has the bits fsadam_plan_step gives for a host float of
+ * the same value.  No counterpart in the reference, whose grad_scale is a host float
+ * (fused_adam_cuda.cpp:4, fused_adam_cuda_kernel.cu:143). */
+int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, const float* grad_scale_dev,
+                               float optim_scale, float decay, int step, int eps_mode, int bias_correction,
+                               float* found_inf_dev, void* hip_stream);
+
 /* Host-only planning (no device needed): how the list would be laid out under the current options.
  * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large.  vector_ok[n_tensors] (may be
  * NULL): 1 = every stream aligned to its 64/128-bit vector. */

@@ -373,6 +373,28 @@ def test_scale_keyword_divides_the_gradients(oracle, api, cuda_device):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("precision_name", ["FULL_PRECISION", "MIXED_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION", "PURE_FP16"])
+@pytest.mark.parametrize("scale", [64.0, 3.0])
+def test_scale_as_a_device_tensor_gives_the_bits_of_a_host_scale(api, cuda_device, precision_name, scale):
+    """step(scale=tensor): the kernel reads the value when it runs and divides by it; a power of two or not,
+    the results are those of step(scale=float)."""
+    Adam, _, Precision = api
+    results = []
+    for on_device in (False, True):
+        params = _random_problem(precision_name, cuda_device, sizes=(10, 3000, 200001), seed=9)
+        opt = Adam(params, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name])
+        holder = torch.zeros(1, device=cuda_device)
+        for step in range(1, 4):
+            _set_grads(params, step, seed=9)
+            holder.fill_(scale)  # written on the stream just before the step: nothing waits on the host
+            opt.step(scale=holder if on_device else scale)
+        results.append([p.detach().clone() for p in params] + [opt.state[p][k].clone() for p in params for k in ("exp_avg", "exp_avg_sq")])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match="float32"):
+        opt.step(scale=torch.ones(1, dtype=torch.float64, device=cuda_device))
+
+
 def test_attached_fp16_copies_follow_the_fp32_parameters(api, cuda_device):
     """attach_fp16_copies: the step leaves half(p) in the attached tensors, parameters and state are those
     of a plain FULL_PRECISION optimizer bit for bit; detaching stops the writes."""

@@ -225,6 +225,10 @@ def test_plan_lifecycle_without_a_device():
     assert L.fsadam_plan_step(handle, 1e-3, 0.9, 0.999, 1e-8, 1.0, 65536.0, 0.0, 1, 1, 1, None, None) == EINVAL
     assert "no tensors" in last_error()
     assert L.fsadam_plan_set_tensors(handle, None, 1, None) == EINVAL
+    # the variant with the gradient scale on the device insists on a pointer
+    assert L.fsadam_plan_step_dev_scale(handle, 1e-3, 0.9, 0.999, 1e-8, None, 65536.0, 0.0, 1, 1, 1, None, None) == EINVAL
+    assert "grad_scale_dev" in last_error()
+    assert L.fsadam_plan_step_dev_scale(None, 1e-3, 0.9, 0.999, 1e-8, ctypes.c_void_p(4096), 65536.0, 0.0, 1, 1, 1, None, None) == EINVAL
     _cabi.check(L.fsadam_plan_destroy(handle))
     _cabi.check(L.fsadam_plan_destroy(None))
     _cabi.check(L.fsadam_clear_cache())

@@ -270,6 +270,35 @@ def test_folding_the_clip_into_the_step_matches_clipping_in_float32(cuda_device)
     assert torch.allclose(outs[0][1], outs[1][1], rtol=1e-6, atol=1e-9)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("max_norm", [1.0, 1e6])
+def test_clip_factor_kept_on_the_device_gives_the_bits_of_the_host_fold(cuda_device, dtype, max_norm):
+    """fold="device": the factor never visits the host; the step kernel reads it from the tensor.  Same
+    value as fold=True computes on the host, hence the same parameters bit for bit; with a max_norm
+    above the norm the factor is exactly 1."""
+    from fairscale_amd.optim import Adam, Precision, clip_grad_norm_
+
+    torch.manual_seed(6)
+    base = (torch.randn(300001, device=cuda_device) * 0.02).to(dtype)
+    grad = (torch.randn(300001, device=cuda_device) * 0.1).to(dtype)
+    precision = Precision.FULL_PRECISION if dtype == torch.float32 else Precision.MEMORY_EFFICIENT_MIXED_PRECISION
+    outs = []
+    for fold in (True, "device"):
+        p = torch.nn.Parameter(base.clone())
+        p.grad = grad.clone()
+        opt = Adam([p], lr=1e-3, precision=precision)
+        norm, scale = clip_grad_norm_([p], max_norm, fold=fold)
+        if fold == "device":
+            assert isinstance(scale, torch.Tensor) and scale.dtype == torch.float32 and scale.shape == (1,) and scale.is_cuda
+        opt.step(scale=scale)
+        outs.append((norm.item(), float(scale), p.detach().clone(), opt.state[p]["exp_avg"].clone(), opt.state[p]["exp_avg_sq"].clone()))
+    # the host factor is a Python float that the call narrows to float32; the device one already is float32
+    assert outs[0][0] == outs[1][0] and float(np.float32(outs[0][1])) == outs[1][1]
+    assert (outs[0][1] > 1.0) == (max_norm == 1.0)
+    for a, b in zip(outs[0][2:], outs[1][2:]):
+        assert torch.equal(a, b)
+
+
 def test_grad_scaler_unscales_through_the_fused_pass(cuda_device):
     from fairscale_amd.optim import Adam, GradScaler, Precision
 
