@@ -85,14 +85,14 @@ struct Options {
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
 // about 40-48 KiB of loads in flight per compute unit, i.e. 10 waves of the 4 KiB-per-wave modes and
-// 12 of the 3-3.5 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
+// 12-13 of the 3-4 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
 int64_t default_lds_throttle(int mode) {
     switch (mode) {
         case FSADAM_FULL_PRECISION: return 16384;
         case FSADAM_FULL_PRECISION_FP16_COPY: return 16384;
         case FSADAM_MIXED_PRECISION: return 15360;
         case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
-        default: return 13312;
+        default: return 12288;
     }
 }
 Options g_opt;

@@ -112,7 +112,7 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "groups"        vectors per lane per stream: 1 or 2 (default 1)
  *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
  *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
- *                   per-mode default (13-16 KiB, default)
+ *                   per-mode default (12-16 KiB, default)
  *   "xcd_remap"     0: tiles in dispatch order (default); R > 0: regroup so that each of the eight XCDs
  *                   takes runs of R consecutive tiles (a very large R gives each XCD one contiguous eighth)
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
