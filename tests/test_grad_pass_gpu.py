@@ -113,6 +113,26 @@ def test_random_gradient_lists_match_the_oracle(cuda_device, seed):
     check(host, dev, stats, want, f"seed {seed}")
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("items,throttle", [(2, 0), (4, 65536), (8, 13312), (8, 0)])
+def test_every_compiled_shape_of_the_pass_matches_the_oracle(cuda_device, dtype, items, throttle):
+    """2, 4 or 8 vectors per lane are compiled; which one runs is picked by the kind of pass unless the
+    options say otherwise.  Same results for all of them."""
+    from fairscale_amd import _cabi
+
+    old = {k: _cabi.get_option(k) for k in ("grad_items", "grad_lds_throttle")}
+    try:
+        _cabi.set_option("grad_items", items)
+        _cabi.set_option("grad_lds_throttle", throttle)
+        for write_back in (False, True):
+            host = host_grads(dtype, 12, SIZES, scale=3.0)
+            dev, stats, want = run_both(host, cuda_device, 1.0 / 3, write_back, misalign=1)
+            check(host, dev, stats, want, f"items {items} throttle {throttle} wb {write_back}")
+    finally:
+        for k, v in old.items():
+            _cabi.set_option(k, v)
+
+
 def test_unscale_by_an_inexact_factor_rounds_twice_on_every_path(cuda_device):
     """half(float32(float(g) * inv_scale)): the float32 rounding comes first, as in torch's kernel.  Many
     tensors just below one tile (element-wise path) plus a large one (vector path), enough elements for

@@ -242,6 +242,44 @@ def test_pure_fp16_odd_optim_scale_rounds_twice_on_every_path(oracle, cuda_devic
              grad_scale=3.0, optim_scale=1000.0)
 
 
+@pytest.fixture
+def options():
+    """Set tuning options for one test and put the defaults back afterwards."""
+    from fairscale_amd import _cabi
+
+    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors")
+    old = {k: _cabi.get_option(k) for k in names}
+
+    def set_many(**kw):
+        for k, v in kw.items():
+            _cabi.set_option(k, v)
+
+    yield set_many
+    for k, v in old.items():
+        _cabi.set_option(k, v)
+
+
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+@pytest.mark.parametrize("block,groups", [(64, 2), (128, 1), (128, 2), (256, 1), (256, 2)])
+def test_every_compiled_tile_shape_matches_the_oracle(oracle, cuda_device, options, mode, block, groups):
+    """The library is built with six workgroup shapes per mode; the default is one wave and one vector per
+    stream.  The others are reachable through the options and must give the same bits."""
+    options(block=block, groups=groups)
+    tile = block * (8 if mode == PURE16 else 4) * groups
+    sizes = [1, tile - 1, tile, tile + 1, 3 * tile + 5, 131072, 131073, 300001]
+    run_case(oracle, cuda_device, mode, sizes, 2, 4800 + mode, dict(DEFAULT, decay=0.01), grad_scale=1.0 if mode == FULL else 8.0,
+             optim_scale=65536.0 if mode == PURE16 else 1.0, misalign={"p": 1})
+
+
+@pytest.mark.parametrize("setting", [dict(xcd_remap=1), dict(xcd_remap=7), dict(xcd_remap=1 << 20), dict(lds_throttle=0),
+                                     dict(lds_throttle=65536), dict(max_large_chunk=4096), dict(max_large_chunk=65536, block=256, groups=2)])
+def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, options, setting):
+    options(**setting)
+    for mode in (MEMEFF, PURE16):
+        run_case(oracle, cuda_device, mode, [5, 4099, 40000, 140001, 524288 + 17], 2, 4900 + mode, DEFAULT, grad_scale=8.0,
+                 optim_scale=65536.0 if mode == PURE16 else 1.0)
+
+
 def test_zero_sized_tensors_in_list(oracle, cuda_device):
     run_case(oracle, cuda_device, FULL, [0, 5, 0, 0, 20000, 0], 2, 4300, DEFAULT)
 
