@@ -280,6 +280,24 @@ def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, opti
                  optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
+def test_more_lists_than_the_table_cache_holds(oracle, cuda_device):
+    """``adam`` keeps the device tables of the last few lists it saw.  Twelve lists stepped in turn, three
+    rounds, two modes: tables are evicted and rebuilt all the time, results stay those of the oracle."""
+    cases = []
+    for k in range(12):
+        mode = MEMEFF if k % 2 else FULL
+        host = C.Tensors(mode, [17 + k, 4096 + k, 140000 + 3 * k], 5000 + k)
+        cases.append((host, GpuList(host, cuda_device), np.zeros(1, np.float32)))
+    for step in (1, 2, 3):
+        for host, dev, flag in cases:
+            grads = host.grads(step)
+            kw = dict(DEFAULT, step=step, grad_scale=1.0, optim_scale=1.0)
+            dev.step(grads, **kw)
+            oracle_step(oracle, host, grads, flag, **kw)
+    for k, (host, dev, _) in enumerate(cases):
+        compare(host, dev, f"list {k}")
+
+
 def test_zero_sized_tensors_in_list(oracle, cuda_device):
     run_case(oracle, cuda_device, FULL, [0, 5, 0, 0, 20000, 0], 2, 4300, DEFAULT)
 
