@@ -280,6 +280,30 @@ def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, opti
                  optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
+def test_pointer_changes_while_earlier_steps_are_in_flight(oracle, cuda_device):
+    """Twelve steps enqueued back to back, each with gradient tensors at new addresses and nothing waiting
+    in between: every step uploads a new table into the next slot of the plan's ring while the kernels
+    of the steps before may still be reading theirs."""
+    from fairscale_amd import fused_adam_hip
+    from fairscale_amd import _cabi
+
+    host = C.Tensors(MEMEFF, [300, 70001, 1 << 21, 5_000_000], 5300)
+    dev = GpuList(host, cuda_device)
+    all_grads = [host.grads(step) for step in range(1, 13)]
+    on_device = [to_gpu(g, cuda_device) for g in all_grads]
+    plan = fused_adam_hip.TensorListPlan(_cabi.MEMORY_EFFICIENT_MIXED_PRECISION, cuda_device)
+    torch.cuda.synchronize(cuda_device)
+    for step, g in enumerate(on_device, start=1):
+        plan.step([dev.p, dev.m, dev.v, g], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, None, step, 1, 1, 0.0)
+    assert plan.info()["uploads"] == 12
+    torch.cuda.synchronize(cuda_device)
+    flag = np.zeros(1, np.float32)
+    for step, grads in enumerate(all_grads, start=1):
+        oracle_step(oracle, host, grads, flag, **dict(DEFAULT, step=step, grad_scale=1.0, optim_scale=1.0))
+    compare(host, dev, "12 steps in flight")
+    plan.close()
+
+
 def test_more_lists_than_the_table_cache_holds(oracle, cuda_device):
     """``adam`` keeps the device tables of the last few lists it saw.  Twelve lists stepped in turn, three
     rounds, two modes: tables are evicted and rebuilt all the time, results stay those of the oracle."""
