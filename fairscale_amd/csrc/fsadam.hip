@@ -81,6 +81,7 @@ struct Options {
     int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
     int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
     int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
+    int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -422,6 +423,7 @@ struct GradPlan {
     int64_t lds_throttle = 0;
     int64_t max_large_chunk = kMaxLargeChunk;
     int64_t unaligned_vectors = 1;
+    int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
     std::vector<FsGradTensor> rows;
     Layout layout;
     TableSlot slots[kTableSlots];
@@ -478,8 +480,10 @@ void grad_plan_free(GradPlan* plan) {
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
-void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors) {
+void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    // a pass that only reads pays for every small store it makes: 16 tiles share one partial
+    *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
     *max_large_chunk = g_opt.max_large_chunk;
     *unaligned_vectors = g_opt.unaligned_vectors;
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
@@ -567,25 +571,35 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     if (rc) return rc;
     rc = order_after(plan->last_use, plan->used, plan->last_stream, stream);  // the partial sums are shared by every call
     if (rc) return rc;
-#define FS_GRAD_LAUNCH(ITEMS)                                                                                               \
-    do {                                                                                                                    \
-        if (n_blocks > 0)                                                                                                   \
-            hipLaunchKernelGGL((fsadam_grad_tiles<T, 64, ITEMS>), dim3((uint32_t)n_blocks), dim3(64), lds, stream,          \
-                               slot.d_table, (uint32_t)log2k, (uint32_t)large_blocks, (uint32_t)L.n_large_descs, inv_scale, \
-                               inv_scale_dev, write_back, first);                                                           \
+    // workgroups of `waves` consecutive tiles, one partial each
+    const int64_t waves = plan->waves;
+    const int64_t n_groups = ceil_div(n_blocks, waves);
+#define FS_GRAD_LAUNCH(WAVES, ITEMS)                                                                                          \
+    hipLaunchKernelGGL((fsadam_grad_tiles<T, WAVES, ITEMS>), dim3((uint32_t)n_groups), dim3(64 * WAVES), lds, stream,        \
+                       slot.d_table, (uint32_t)log2k, (uint32_t)large_blocks, (uint32_t)L.n_large_descs, (uint32_t)n_blocks, \
+                       inv_scale, inv_scale_dev, write_back, first)
+#define FS_GRAD_ITEMS(WAVES)                          \
+    do {                                              \
+        if (plan->items == 2) FS_GRAD_LAUNCH(WAVES, 2);      \
+        else if (plan->items == 8) FS_GRAD_LAUNCH(WAVES, 8); \
+        else FS_GRAD_LAUNCH(WAVES, 4);                       \
     } while (0)
     const size_t lds = (size_t)plan->lds_throttle;
-    if (plan->items == 2) FS_GRAD_LAUNCH(2);
-    else if (plan->items == 8) FS_GRAD_LAUNCH(8);
-    else FS_GRAD_LAUNCH(4);
+    if (n_blocks > 0) {
+        if (waves == 16) FS_GRAD_ITEMS(16);
+        else if (waves == 4) FS_GRAD_ITEMS(4);
+        else FS_GRAD_ITEMS(1);
+    }
+#undef FS_GRAD_ITEMS
 #undef FS_GRAD_LAUNCH
     FS_HIP(hipGetLastError());
-    // two fixed-shape reduction steps, then publish (also when the list holds no element: everything is zero)
-    const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_blocks, 1024)));
-    const uint32_t per_block = (uint32_t)ceil_div(std::max<int64_t>(n_blocks, 1), blocks2);
-    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_blocks, per_block, second);
-    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total);
-    hipLaunchKernelGGL(fsadam_grad_publish, dim3(1), dim3(64), 0, stream, total, (int)(sizeof(T) == 2), found_inf, sum_squares, abs_max);
+    // two fixed-shape reduction steps, the second of which publishes (also when the list holds no element: everything is zero)
+    const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_groups, 1024)));
+    const uint32_t per_block = (uint32_t)ceil_div(std::max<int64_t>(n_groups, 1), blocks2);
+    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_groups, per_block, second, 0, 0,
+                       (float*)nullptr, (double*)nullptr, (float*)nullptr);
+    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total, 1, (int)(sizeof(T) == 2),
+                       found_inf, sum_squares, abs_max);
     FS_HIP(hipGetLastError());
     rc = slot_mark(slot, stream);
     if (rc) return rc;
@@ -670,6 +684,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "grad_items") {
         if (value != 0 && value != 2 && value != 4 && value != 8) return fail(FSADAM_EINVAL, "grad_items must be 0 (automatic), 2, 4 or 8");
         g_opt.grad_items = value;
+    } else if (k == "grad_waves") {
+        if (value != 0 && value != 1 && value != 4 && value != 16) return fail(FSADAM_EINVAL, "grad_waves must be 0 (automatic), 1, 4 or 16");
+        g_opt.grad_waves = value;
     } else if (k == "grad_lds_throttle") {
         if (value < -1 || value > 65536) return fail(FSADAM_EINVAL, "grad_lds_throttle must be -1 (automatic) or in [0, 65536] bytes");
         g_opt.grad_lds_throttle = value;
@@ -691,6 +708,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
+    else if (k == "grad_waves") *value = g_opt.grad_waves;
     else return fail(FSADAM_EINVAL, "unknown option '" + k + "'");
     return FSADAM_OK;
 }
@@ -845,14 +863,15 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned;
-    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned);
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves;
+    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
+               &cur_waves);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -877,6 +896,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->lds_throttle = cur_lds;
         victim->max_large_chunk = cur_chunk;
         victim->unaligned_vectors = cur_unaligned;
+        victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;

@@ -55,9 +55,12 @@ __device__ __forceinline__ uint32_t max_u16x2(uint32_t a, uint32_t b) {
 // half); or through float.
 enum : int { kGradUnit = 0, kGradHalfScale = 1, kGradFloatScale = 2 };
 
+// Only the largest incoming magnitude is tracked per element.  The largest STORED magnitude follows
+// from it: g -> dtype(g * inv_scale) is a multiplication by a constant followed by roundings, all
+// monotone in |g|, so the maximum of the results is the result of the maximum (NaN stays NaN, an
+// overflow stays inf).  It is formed once per wave after the reduction.
 struct GradAcc {
     float sum = 0.f;
-    uint32_t stored_max = 0;
     uint32_t incoming_max = 0;
 };
 
@@ -73,7 +76,6 @@ __device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2
         r[1] = (_Float16)as_float32((float)r[1] * inv_scale);
     }
     const uint32_t out = __builtin_bit_cast(uint32_t, r);
-    if (HOW != kGradUnit) acc.stored_max = max_u16x2(acc.stored_max, out & 0x7fff7fffu);
     // fused multiply-adds with half operands widened on the fly (v_fma_mix_f32): the product of two
     // halves is exact in fp32, subnormal halves included
     acc.sum = __builtin_fmaf((float)r[0], (float)r[0], acc.sum);
@@ -94,10 +96,6 @@ __device__ __forceinline__ float grad_float(float g, float inv_scale, GradAcc& a
     const uint32_t mag = __builtin_bit_cast(uint32_t, g) & 0x7fffffffu;
     acc.incoming_max = mag > acc.incoming_max ? mag : acc.incoming_max;
     const float r = (HOW == kGradUnit) ? g : g * inv_scale;
-    if (HOW != kGradUnit) {
-        const uint32_t rm = __builtin_bit_cast(uint32_t, r) & 0x7fffffffu;
-        acc.stored_max = rm > acc.stored_max ? rm : acc.stored_max;
-    }
     acc.sum += r * r;
     return r;
 }
@@ -106,8 +104,9 @@ __device__ __forceinline__ float grad_scalar(float g, int how, float inv_scale, 
     return how == kGradUnit ? grad_float<kGradUnit>(g, inv_scale, acc) : grad_float<kGradFloatScale>(g, inv_scale, acc);
 }
 
+// One wave's tile: BLOCK = 64 lanes, `lane` this thread's position in it.
 template <typename T, int BLOCK, int ITEMS, int HOW, bool WRITE>
-__device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, float inv_scale, GradAcc& acc) {
+__device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint32_t lane, float inv_scale, GradAcc& acc) {
     constexpr int E = GradTraits<T>::kElems;
     constexpr uint32_t kTile = BLOCK * E * ITEMS;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -118,7 +117,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, floa
         u32x4 raw[ITEMS];
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
-            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
+            raw[k] = __builtin_nontemporal_load(reinterpret_cast<gptr<const u32x4_in_memory>>(g + (k * BLOCK + lane) * E));
         const f16x2 inv_half = {(_Float16)inv_scale, (_Float16)inv_scale};
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k) {
@@ -131,64 +130,104 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, floa
                 else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
             }
             if (WRITE && HOW != kGradUnit)
-                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + threadIdx.x) * E));
+                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + lane) * E));
         }
     } else {
         const uint32_t count = left < kTile ? left : kTile;
-        for (uint32_t e = threadIdx.x; e < count; e += BLOCK) {
+        for (uint32_t e = lane; e < count; e += BLOCK) {
             const T r = grad_scalar(g[e], HOW, inv_scale, acc);
             if (WRITE && HOW != kGradUnit) g[e] = r;
         }
     }
 }
 
-template <typename T, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
-                                                           uint32_t n_large_descs, float inv_scale_value,
-                                                           const float* __restrict__ inv_scale_dev, int write_back,
-                                                           GradPartial* __restrict__ partials) {
-    static_assert(BLOCK == 64, "one wave per workgroup: the partial is reduced with wave shuffles only");
+// One wave = one tile of 64 x ITEMS 16-byte vectors, found through the table like the tiles of the
+// Adam step.  A workgroup is WAVES consecutive tiles and writes ONE partial: in a pass that only
+// reads, every small store forces a read/write turnaround somewhere in the DRAM, and one 16-byte
+// store per wave (400 000 of them over the benchmark's shard) was measured to cost 5-8 % of the read
+// bandwidth; with 16 waves per workgroup the cost is gone.  `n_tiles`: tiles really there (the last
+// workgroup may have fewer than WAVES).
+template <typename T, int WAVES, int ITEMS>
+__global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
+                                                                uint32_t n_large_descs, uint32_t n_tiles, float inv_scale_value,
+                                                                const float* __restrict__ inv_scale_dev, int write_back,
+                                                                GradPartial* __restrict__ partials) {
+    constexpr int BLOCK = 64;
     constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
-    const uint32_t block = blockIdx.x;
-    const bool large = block < n_large_blocks;  // uniform: scalar selects
-    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
-    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
-    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
-    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
-        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
-    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    // the wave's number within the workgroup is the same for all its lanes: say so, and the tile's
+    // descriptor stays a scalar load
+    const uint32_t wave = WAVES == 1 ? 0u : (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t lane = WAVES == 1 ? threadIdx.x : (threadIdx.x & 63u);
+    const uint32_t block = blockIdx.x * WAVES + wave;
     // the scale may live on the device (a loss scaler keeps it there): uniform address, scalar load
     const float inv_scale = inv_scale_dev ? *(const __attribute__((address_space(4))) float*)inv_scale_dev : inv_scale_value;
+    const bool half_scale = sizeof(T) == 2 && (float)(_Float16)inv_scale == inv_scale;
 
     GradAcc acc;
-    if (off < d.n) {
-        if (inv_scale == 1.0f) {
-            grad_tile<T, BLOCK, ITEMS, kGradUnit, false>(d, off, inv_scale, acc);
-        } else if (sizeof(T) == 2 && (float)(_Float16)inv_scale == inv_scale) {
-            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradHalfScale, true>(d, off, inv_scale, acc);
-            else grad_tile<T, BLOCK, ITEMS, kGradHalfScale, false>(d, off, inv_scale, acc);
-        } else {
-            if (write_back) grad_tile<T, BLOCK, ITEMS, kGradFloatScale, true>(d, off, inv_scale, acc);
-            else grad_tile<T, BLOCK, ITEMS, kGradFloatScale, false>(d, off, inv_scale, acc);
+    bool any = false;  // uniform within the wave
+    if (block < n_tiles) {
+        const bool large = block < n_large_blocks;  // uniform: scalar selects
+        const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
+        const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
+        typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
+        const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
+            (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
+        const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+        any = off < d.n;
+        if (any) {
+            if (inv_scale == 1.0f) {
+                grad_tile<T, BLOCK, ITEMS, kGradUnit, false>(d, off, lane, inv_scale, acc);
+            } else if (half_scale) {
+                if (write_back) grad_tile<T, BLOCK, ITEMS, kGradHalfScale, true>(d, off, lane, inv_scale, acc);
+                else grad_tile<T, BLOCK, ITEMS, kGradHalfScale, false>(d, off, lane, inv_scale, acc);
+            } else {
+                if (write_back) grad_tile<T, BLOCK, ITEMS, kGradFloatScale, true>(d, off, lane, inv_scale, acc);
+                else grad_tile<T, BLOCK, ITEMS, kGradFloatScale, false>(d, off, lane, inv_scale, acc);
+            }
         }
-        if (inv_scale == 1.0f) acc.stored_max = acc.incoming_max;  // nothing was rescaled
     }
-    if (sizeof(T) == 2) {  // unpack the two 16-bit maxima
-        acc.stored_max = (acc.stored_max & 0xffffu) > (acc.stored_max >> 16) ? (acc.stored_max & 0xffffu) : (acc.stored_max >> 16);
+    if (sizeof(T) == 2)  // unpack the two 16-bit maxima
         acc.incoming_max = (acc.incoming_max & 0xffffu) > (acc.incoming_max >> 16) ? (acc.incoming_max & 0xffffu) : (acc.incoming_max >> 16);
-    }
     // wave reduction in a fixed order (xor butterfly): the same inputs always give the same bits
     double dsum = (double)acc.sum;
-    uint32_t smax = acc.stored_max, imax = acc.incoming_max;
+    uint32_t imax = acc.incoming_max;
 #pragma unroll
     for (int w = 32; w >= 1; w >>= 1) {
         dsum += __shfl_xor(dsum, w, 64);
-        const uint32_t s2 = (uint32_t)__shfl_xor((int)smax, w, 64), i2 = (uint32_t)__shfl_xor((int)imax, w, 64);
-        smax = s2 > smax ? s2 : smax;
+        const uint32_t i2 = (uint32_t)__shfl_xor((int)imax, w, 64);
         imax = i2 > imax ? i2 : imax;
     }
+    // what the largest magnitude becomes when it is unscaled and stored (see GradAcc)
+    uint32_t smax = imax;
+    if (any && inv_scale != 1.0f) {
+        if (sizeof(T) == 2) {
+            const _Float16 top = __builtin_bit_cast(_Float16, (uint16_t)imax);
+            const _Float16 r = half_scale ? top * (_Float16)inv_scale : (_Float16)as_float32((float)top * inv_scale);
+            smax = __builtin_bit_cast(uint16_t, r) & 0x7fffu;
+        } else {
+            smax = __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, imax) * inv_scale) & 0x7fffffffu;
+        }
+    }
+    if (WAVES > 1) {  // the workgroup's waves, added in wave order by one thread
+        __shared__ double s_sum[WAVES];
+        __shared__ uint32_t s_stored[WAVES], s_incoming[WAVES];
+        if (lane == 0) {
+            s_sum[wave] = dsum;
+            s_stored[wave] = smax;
+            s_incoming[wave] = imax;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) {
+                dsum += s_sum[w];
+                smax = s_stored[w] > smax ? s_stored[w] : smax;
+                imax = s_incoming[w] > imax ? s_incoming[w] : imax;
+            }
+        }
+    }
     if (threadIdx.x == 0) {
-        gptr<GradPartial> out = (gptr<GradPartial>)partials + block;
+        gptr<GradPartial> out = (gptr<GradPartial>)partials + blockIdx.x;
         out->sum_squares = dsum;
         out->stored_max = smax;
         out->incoming_max = imax;
@@ -196,9 +235,11 @@ __global__ __launch_bounds__(BLOCK) void fsadam_grad_tiles(const ChunkDesc* __re
 }
 
 // Fixed-order reduction of `n` partials into `out[blockIdx.x]`: block b takes the b-th contiguous
-// slice, thread t every 256th entry of it, then a shared-memory tree.
+// slice, thread t every 256th entry of it, then a shared-memory tree.  The last step (one block,
+// `publish` set) hands the result to the caller's three outputs instead.
 __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
-                                                          GradPartial* __restrict__ out) {
+                                                          GradPartial* __restrict__ out, int publish, int is_half,
+                                                          float* found_inf, double* sum_squares, float* abs_max) {
     __shared__ double s_sum[256];
     __shared__ uint32_t s_stored[256];
     __shared__ uint32_t s_incoming[256];
@@ -222,23 +263,17 @@ __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __r
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) {
+    if (threadIdx.x != 0) return;
+    if (!publish) {
         out[blockIdx.x].sum_squares = s_sum[0];
         out[blockIdx.x].stored_max = s_stored[0];
         out[blockIdx.x].incoming_max = s_incoming[0];
+        return;
     }
-}
-
-// Hands the single remaining partial to the caller's three outputs.
-__global__ void fsadam_grad_publish(const GradPartial* __restrict__ total, int is_half, float* found_inf, double* sum_squares,
-                                    float* abs_max) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
-        if (total->incoming_max >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
-        if (sum_squares) *sum_squares = total->sum_squares;
-        if (abs_max)
-            *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)total->stored_max) : __builtin_bit_cast(float, total->stored_max);
-    }
+    const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
+    if (s_incoming[0] >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
+    if (sum_squares) *sum_squares = s_sum[0];
+    if (abs_max) *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)s_stored[0]) : __builtin_bit_cast(float, s_stored[0]);
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));

@@ -118,6 +118,8 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
  *                   4 for one that writes the gradients back (default 0)
  *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
+ *   "grad_waves"    gradient pass: tiles (one wave each) per workgroup, 1, 4 or 16; the workgroup writes one
+ *                   partial result.  0 = 16 for a read-only pass, 1 for one that writes back (default 0)
  *   "unaligned_vectors"  1 (default): full tiles of a tensor whose streams are only element-aligned (a view that
  *                   starts at an odd element) still move with 64/128-bit vector instructions; 0: such tensors
  *                   are processed element by element (measured 1.5-2x slower)

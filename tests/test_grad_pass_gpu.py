@@ -114,16 +114,17 @@ def test_random_gradient_lists_match_the_oracle(cuda_device, seed):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("items,throttle", [(2, 0), (4, 65536), (8, 13312), (8, 0)])
-def test_every_compiled_shape_of_the_pass_matches_the_oracle(cuda_device, dtype, items, throttle):
-    """2, 4 or 8 vectors per lane are compiled; which one runs is picked by the kind of pass unless the
-    options say otherwise.  Same results for all of them."""
+@pytest.mark.parametrize("items,throttle,waves", [(2, 0, 1), (4, 65536, 4), (8, 13312, 16), (8, 0, 1), (2, 0, 16), (4, 0, 16), (8, 8192, 4)])
+def test_every_compiled_shape_of_the_pass_matches_the_oracle(cuda_device, dtype, items, throttle, waves):
+    """2, 4 or 8 vectors per lane and 1, 4 or 16 waves per workgroup are compiled; which runs is picked by
+    the kind of pass unless the options say otherwise.  Same results for all of them."""
     from fairscale_amd import _cabi
 
-    old = {k: _cabi.get_option(k) for k in ("grad_items", "grad_lds_throttle")}
+    old = {k: _cabi.get_option(k) for k in ("grad_items", "grad_lds_throttle", "grad_waves")}
     try:
         _cabi.set_option("grad_items", items)
         _cabi.set_option("grad_lds_throttle", throttle)
+        _cabi.set_option("grad_waves", waves)
         for write_back in (False, True):
             host = host_grads(dtype, 12, SIZES, scale=3.0)
             dev, stats, want = run_both(host, cuda_device, 1.0 / 3, write_back, misalign=1)
