@@ -291,3 +291,28 @@ def test_optimizer_module_imports_and_exposes_the_reference_names():
     assert [p.value for p in fo.Precision] == [1, 2, 3, 4]  # auto() values of adam.py:19-23
     assert issubclass(fo.Adam, torch.optim.Optimizer)
     assert issubclass(fo.GradScaler, torch.amp.GradScaler)
+
+
+def test_versioned_state_map_counts_what_changes_the_key_set():
+    """``optimizer.state`` of Adam: the steady-state step trusts its cached per-parameter state dicts only
+    while this counter stands still."""
+    import copy
+    import pickle
+
+    from fairscale_amd.optim.adam import _VersionedState
+
+    st = _VersionedState(dict)
+    v0 = st.version
+    a = st["a"]           # created on first access (torch's defaultdict(dict) behaviour)
+    assert a == {} and st.version > v0
+    v1 = st.version
+    st["a"]["step"] = 1   # changing a state dict in place is not a change of the map
+    assert st["a"] is a and st.version == v1
+    for change in (lambda: st.__setitem__("b", {}), lambda: st.pop("b"), lambda: st.setdefault("c", {}), lambda: st.update(d={}),
+                   lambda: st.__delitem__("c"), lambda: st.popitem(), lambda: st.clear()):
+        before = st.version
+        change()
+        assert st.version > before
+    st["x"]["step"] = 7
+    for clone in (pickle.loads(pickle.dumps(st)), copy.deepcopy(st)):
+        assert type(clone) is _VersionedState and clone["x"] == {"step": 7} and clone["fresh"] == {}
