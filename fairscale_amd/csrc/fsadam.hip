@@ -246,6 +246,17 @@ int slot_mark(TableSlot& slot, hipStream_t stream) {
     return FSADAM_OK;
 }
 
+// The scalars of a step (step size, scales) travel by value in the kernel arguments and the table slots
+// are guarded by events the host waits on: recorded into a HIP graph, every replay would repeat the
+// first step's bias correction and the events could never be waited for.  Refuse instead of going wrong.
+int refuse_capture(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    FS_HIP(hipStreamIsCapturing(stream, &status));
+    if (status != hipStreamCaptureStatusNone)
+        return fail(FSADAM_EINVAL, "the stream is being captured into a graph: this call cannot be recorded (its step-dependent scalars are kernel arguments)");
+    return FSADAM_OK;
+}
+
 void plan_release_buffers(FsAdamPlan* plan) {
     for (TableSlot& slot : plan->slots) slot_release(slot);
     plan->current = -1;
@@ -318,6 +329,8 @@ int launch_mode(int mode, const ChunkDesc* table, int64_t n_large_descs, int64_t
 int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, hipStream_t stream) {
     int rc = validate_rows(tensors, n, plan->mode);
     if (rc) return rc;
+    rc = refuse_capture(stream);
+    if (rc) return rc;
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     if (plan->device != dev) {
@@ -384,6 +397,7 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     if (eps_mode != FSADAM_EPS_INSIDE_SQRT && eps_mode != FSADAM_EPS_OUTSIDE_SQRT)
         return fail(FSADAM_EINVAL, "eps_mode must be 0 (inside sqrt) or 1 (outside)");
     if (plan->mode == FSADAM_PURE_FP16 && !found_inf) return fail(FSADAM_EINVAL, "PURE_FP16 needs a found_inf device pointer");
+    if (int refused = refuse_capture(stream)) return refused;
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     if (dev != plan->device)
@@ -863,6 +877,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
     int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves;
     grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
                &cur_waves);

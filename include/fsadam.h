@@ -144,7 +144,11 @@ int fsadam_get_option(const char* name, int64_t* value);
  * hip_stream        : hipStream_t to enqueue on (NULL = the default stream).
  *
  * The device-side tensor table is cached inside the library, keyed on the contents of `tensors`;
- * an unchanged list costs no upload. */
+ * an unchanged list costs no upload.
+ *
+ * Not recordable into a HIP graph: the step size depends on `step` and travels by value, so a replay
+ * would repeat the recorded step's bias correction.  A call on a stream that is being captured
+ * returns FSADAM_EINVAL and enqueues nothing (the same holds for the plan calls and the gradient pass). */
 int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, float lr, float beta1,
                 float beta2, float eps, float grad_scale, float optim_scale, float decay, int step,
                 int eps_mode, int bias_correction, float* found_inf_dev, void* hip_stream);

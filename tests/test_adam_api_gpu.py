@@ -609,3 +609,26 @@ def test_added_param_group_steps_with_its_own_hyperparameters(api, cuda_device):
     assert len(both._plans) == 2
     for p, q in zip(a + b, a2 + b2):
         assert torch.equal(p, q)
+
+
+def test_a_step_on_a_capturing_stream_is_refused(api, cuda_device):
+    """Recorded into a graph the step would replay one step's bias correction for ever: the library says no,
+    enqueues nothing, and the optimizer works on afterwards."""
+    Adam, _, _ = api
+    params = _random_problem("FULL_PRECISION", cuda_device, sizes=(1000, 70001), seed=11)
+    opt = Adam(params, lr=1e-2)
+    _set_grads(params, 1, seed=11)
+    opt.step()
+    torch.cuda.synchronize(cuda_device)
+    before = [p.detach().clone() for p in params]
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="captured"):
+        with torch.cuda.graph(graph):
+            opt.step()
+    torch.cuda.synchronize(cuda_device)
+    for p, b in zip(params, before):
+        assert torch.equal(p, b)
+    assert opt.state[params[0]]["step"] == 2  # the walk had advanced the counters before the native call refused
+    opt.step()
+    torch.cuda.synchronize(cuda_device)
+    assert not torch.equal(params[1], before[1])
