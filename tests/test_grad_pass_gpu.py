@@ -354,3 +354,44 @@ def test_grad_scaler_unscales_through_the_fused_pass(cuda_device):
     scaler.step(opt)
     scaler.update()
     assert torch.equal(w.detach(), before) and scaler.get_scale() == scale_before * 0.5
+
+
+def test_whole_flow_unscale_norm_clip_on_device_step(oracle, cuda_device):
+    """scale(loss).backward() -> unscale_ (fused pass) -> norm from the same pass -> clip factor formed on the
+    device -> step(scale=factor) -> update(): nothing reads a value back between backward and the end of the
+    step.  Replayed on the host from the scaled gradients: same parameters bit for bit."""
+    from fairscale_amd.optim import Adam, GradScaler, Precision
+
+    torch.manual_seed(8)
+    sizes = [(64, 32), (64,), (300, 128)]
+    params = [(torch.randn(*s, device=cuda_device) * 0.1).half().requires_grad_() for s in sizes]
+    x = torch.randn(32, device=cuda_device).half()
+    opt = Adam(params, lr=1e-2, precision=Precision.MEMORY_EFFICIENT_MIXED_PRECISION)
+    ref = oracle.OracleAdam([p.detach().cpu().numpy().reshape(-1).copy() for p in params], oracle.MEMORY_EFFICIENT_MIXED_PRECISION, lr=1e-2)
+    scaler = GradScaler(init_scale=256.0, growth_interval=2)
+    max_norm = 0.05
+    for it in range(5):
+        opt.zero_grad()
+        w, b, w2 = params
+        loss = (w.mv(x) + b).float().pow(2).sum() + w2.float().pow(2).sum() * 0.01
+        scaler.scale(loss).backward()
+        scale_now = scaler.get_scale()
+        scaled = [p.grad.detach().cpu().numpy().reshape(-1).copy() for p in params]
+        scaler.unscale_(opt)
+        norm = scaler.unscaled_grad_norm(opt)
+        assert norm is not None
+        factor = torch.clamp(norm / max_norm, min=1.0).reshape(1)
+        scaler.step(opt, scale=factor)
+        scaler.update()
+        # the same on the host: unscale as the pass stores it, float64 sum of squares, the factor in float32
+        inv = np.float32(1.0 / scale_now)
+        unscaled = [(g.astype(np.float32) * inv).astype(np.float16) for g in scaled]
+        total = np.sqrt(sum(float((u.astype(np.float64) ** 2).sum()) for u in unscaled))
+        device_norm = np.float32(norm.item())  # read back only here, for the replay
+        assert abs(float(device_norm) - total) <= 1e-6 * total, f"iteration {it}"
+        host_factor = max(device_norm / np.float32(max_norm), np.float32(1.0))
+        assert float(factor) == float(host_factor), f"iteration {it}"
+        ref.step(unscaled, scale=float(host_factor))
+        for p, want in zip(params, ref.params):
+            assert np.array_equal(p.detach().cpu().numpy().reshape(-1).view(np.uint16), want.view(np.uint16)), f"iteration {it}"
+    assert scaler.get_scale() > 256.0  # it grew: no overflow was seen
