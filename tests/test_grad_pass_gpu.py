@@ -358,8 +358,9 @@ def test_grad_scaler_unscales_through_the_fused_pass(cuda_device):
 
 def test_whole_flow_unscale_norm_clip_on_device_step(oracle, cuda_device):
     """scale(loss).backward() -> unscale_ (fused pass) -> norm from the same pass -> clip factor formed on the
-    device -> step(scale=factor) -> update(): nothing reads a value back between backward and the end of the
-    step.  Replayed on the host from the scaled gradients: same parameters bit for bit."""
+    device -> step(scale=factor) -> update(): the norm and the clip decision never visit the host (torch's scaler
+    still reads its own overflow flag inside step()).  Replayed on the host from the scaled gradients: same
+    parameters bit for bit."""
     from fairscale_amd.optim import Adam, GradScaler, Precision
 
     torch.manual_seed(8)
