@@ -138,10 +138,13 @@ py::tuple fill_rows(py::list lists, py::tuple dtype_codes, int device, uintptr_t
     return as_tuple(r);
 }
 
-// The steady-state walk of Adam.step: every parameter of the group has a dense gradient and a
-// state {step, exp_avg, exp_avg_sq}.  p comes from `masters` when given (MIXED_PRECISION: the fp32
-// copies, with the fp16 parameters as p_copy), else from `params`; `outs` are attached fp16 copies.
-// When everything checks, each state's step is incremented and the last one is returned.
+// The steady-state walk of Adam.step.  `states[t]` is the state dict {step, exp_avg, exp_avg_sq} of
+// parameter t, or None for a parameter that had no gradient when the lists were collected: such a
+// parameter must still have none (adam.py:214-215 skips it), the others must have a dense one.  p
+// comes from `masters` when given (MIXED_PRECISION: the fp32 copies, with the fp16 parameters as
+// p_copy), else from `params`; `outs` are attached fp16 copies (None where states is None).  Rows are
+// written for the parameters that take part, in order.  When everything checks, each state's step
+// is incremented and the last one is returned.
 //
 // `snapshot` is the tuple of parameter objects `states` was collected for: a list edited in place since
 // then is reported as stale instead of pairing a new parameter with another one's state.
@@ -173,6 +176,7 @@ py::tuple gather(py::list params, py::tuple snapshot, py::object masters, py::li
     const c10::ScalarType g_dtype = dtype_of_code(dtype_codes[2].cast<int>());
     int64_t* rows = reinterpret_cast<int64_t*>(rows_address);
     bool changed = false;
+    int64_t active = 0;  // rows written so far
     auto stop = [&](int status, int64_t list, int64_t index) {
         r.status = status;
         r.list = list;
@@ -188,8 +192,12 @@ py::tuple gather(py::list params, py::tuple snapshot, py::object masters, py::li
             const at::Tensor* p = mixed ? plain_tensor(PyList_GET_ITEM(masters.ptr(), t)) : param;
             if (!p) return stop(kNotTensor, 0, t);
             const at::Tensor& g = param->grad();
-            if (!g.defined()) return stop(kNoGrad, 3, t);
             PyObject* st = PyList_GET_ITEM(states.ptr(), t);
+            if (st == Py_None) {  // sat out when the lists were collected
+                if (g.defined()) return stop(kStale, 3, t);
+                continue;
+            }
+            if (!g.defined()) return stop(kNoGrad, 3, t);
             if (!PyDict_Check(st)) return stop(kNoState, 1, t);
             PyObject* m_obj = PyDict_GetItemWithError(st, k_avg);
             PyObject* v_obj = PyDict_GetItemWithError(st, k_sq);
@@ -207,7 +215,8 @@ py::tuple gather(py::list params, py::tuple snapshot, py::object masters, py::li
             if ((bad = check_tensor(*m, s_dtype, device, numel))) return stop(bad, 1, t);
             if ((bad = check_tensor(*v, s_dtype, device, numel))) return stop(bad, 2, t);
             if ((bad = check_tensor(g, g_dtype, device, numel))) return stop(bad, 3, t);
-            int64_t* row = rows + t * 6;
+            int64_t* row = rows + active * 6;
+            active += 1;
             put(row + 0, reinterpret_cast<int64_t>(p->data_ptr()), &changed);
             put(row + 1, reinterpret_cast<int64_t>(m->data_ptr()), &changed);
             put(row + 2, reinterpret_cast<int64_t>(v->data_ptr()), &changed);
@@ -226,10 +235,12 @@ py::tuple gather(py::list params, py::tuple snapshot, py::object masters, py::li
         r.status = kError;
         return as_tuple(r, py::str(e.what()));
     }
+    if (active == 0) return stop(kNoGrad, 3, 0);
     // everything checked: advance the step counters (adam.py:230)
     PyObject* last = nullptr;
     for (int64_t t = 0; t < n; ++t) {
         PyObject* st = PyList_GET_ITEM(states.ptr(), t);
+        if (st == Py_None) continue;
         PyObject* next = PyNumber_Add(PyDict_GetItemWithError(st, k_step), one);
         if (!next) throw py::error_already_set();
         if (PyDict_SetItem(st, k_step, next) != 0) {

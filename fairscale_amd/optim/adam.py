@@ -255,13 +255,16 @@ class Adam(torch.optim.Optimizer):
         state_map, optim_type = self.state, self.optim_type
         masters = self.fp32_param_groups[gi]["params"] if mixed else None
         batches: Dict[torch.device, List[List[torch.Tensor]]] = {}
-        states: List[dict] = []
+        states: List[Optional[dict]] = []  # one entry per parameter; None for those that sit this step out
+        outs: List[Optional[torch.Tensor]] = []
         step_no = None
         params = group["params"]
         depth = 5 if (mixed or copies is not None) else 4
         for pj, p in enumerate(params):
             grad = p.grad
             if grad is None:
+                states.append(None)
+                outs.append(None)
                 continue
             if grad.is_sparse:
                 raise RuntimeError("FusedAdam does not support sparse gradients, please consider SparseAdam instead")
@@ -281,15 +284,20 @@ class Adam(torch.optim.Optimizer):
             lists[3].append(grad)
             if mixed:
                 lists[4].append(p)
+                outs.append(None)
             elif copies is not None:
                 if p not in copies:
                     raise RuntimeError("a parameter with a gradient has no fp16 copy attached")
                 lists[4].append(copies[p])
+                outs.append(copies[p])
+            else:
+                outs.append(None)
         caches = self.__dict__.setdefault("_group_cache", {})
-        if len(states) == len(params) and len(batches) == 1:
-            device, lists = next(iter(batches.items()))
-            outs = lists[4] if depth == 5 else None
-            caches[gi] = (params, tuple(params), states, masters, outs, device, state_map, state_map.version)
+        if len(batches) == 1:  # one device: the steady-state walks can take over from the next step on
+            device = next(iter(batches))
+            n_active = len(batches[device][0])
+            caches[gi] = (params, tuple(params), states, masters, outs if (copies is not None and not mixed) else None, device, state_map,
+                          state_map.version, n_active)
         else:
             caches.pop(gi, None)
         return batches, step_no
@@ -300,7 +308,7 @@ class Adam(torch.optim.Optimizer):
         cache = self.__dict__.get("_group_cache", {}).get(gi)
         if cache is None:
             return None
-        params, snapshot, states, masters, outs, device, state_map, version = cache
+        params, snapshot, states, masters, outs, device, state_map, version, _ = cache
         if group["params"] is not params or len(params) != len(snapshot) or len(snapshot) == 0:
             return None
         if self.state is not state_map or state_map.version != version:
@@ -319,12 +327,12 @@ class Adam(torch.optim.Optimizer):
         cache = self._steady_group(gi, group)
         if cache is None:
             return None
-        params, snapshot, states, masters, outs, device, _, _ = cache
+        params, snapshot, states, masters, outs, device, _, _, n_active = cache
         if device.type != "cuda":
             return None
         plan = self._plan_for(gi, device, native_mode)
         codes = mode_codes(native_mode)
-        buf = plan.rows_buffer(len(snapshot))
+        buf = plan.rows_buffer(n_active)
         status, _, _, step_no = native.gather(params, snapshot, masters, states, None if masters is not None else outs,
                                                (codes[0], codes[1], codes[3]), device.index, buf.ctypes.data)
         if status < 0:
@@ -345,24 +353,37 @@ class Adam(torch.optim.Optimizer):
         cache = self._steady_group(gi, group)
         if cache is None:
             return None, None
-        params, snapshot, states, masters, outs, device, _, _ = cache
+        params, snapshot, states, masters, outs, device, _, _, _ = cache
         if any(map(is_not, params, snapshot)):
             return None, None  # the list was edited in place: the collected states belong to other parameters
-        grads = [p.grad for p in params]
-        for g in grads:
+        lists: List[List[torch.Tensor]] = [[] for _ in range(5 if (masters is not None or outs is not None) else 4)]
+        taking_part = []
+        for pj, (p, st) in enumerate(zip(params, states)):
+            g = p.grad
+            if st is None:
+                if g is not None:
+                    return None, None  # a parameter that sat out has a gradient now
+                continue
             if g is None or g.is_sparse:
                 return None, None
-        try:
-            m_list = [st["exp_avg"] for st in states]
-            v_list = [st["exp_avg_sq"] for st in states]
-        except KeyError:  # a state dict was emptied behind our back: let the general walk re-initialise it
+            try:
+                lists[1].append(st["exp_avg"])
+                lists[2].append(st["exp_avg_sq"])
+                st["step"]
+            except KeyError:  # a state dict was emptied behind our back: let the general walk re-initialise it
+                return None, None
+            lists[0].append(masters[pj] if masters is not None else p)
+            lists[3].append(g)
+            if masters is not None:
+                lists[4].append(p)
+            elif outs is not None:
+                lists[4].append(outs[pj])
+            taking_part.append(st)
+        if not taking_part:
             return None, None
-        for st in states:
+        for st in taking_part:
             st["step"] += 1
-        lists = [masters if masters is not None else params, m_list, v_list, grads]
-        if outs is not None:
-            lists.append(outs)
-        return {device: lists}, states[-1]["step"]
+        return {device: lists}, taking_part[-1]["step"]
 
     def step(self, closure: Optional[Callable[[], float]] = None, *, scale: Union[float, torch.Tensor] = 1.0) -> Optional[float]:
         """One optimization step (adam.py:184-297).

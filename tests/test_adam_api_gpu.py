@@ -632,3 +632,33 @@ def test_a_step_on_a_capturing_stream_is_refused(api, cuda_device):
     opt.step()
     torch.cuda.synchronize(cuda_device)
     assert not torch.equal(params[1], before[1])
+
+
+@pytest.mark.parametrize("use_helper", [True, False])
+def test_frozen_parameters_do_not_disable_the_steady_state_walk(api, cuda_device, use_helper, monkeypatch):
+    """A parameter that never gets a gradient (a frozen layer left in the list) is skipped as in
+    adam.py:214-215, and the others still go through the cached walk: one table upload, right results;
+    when it starts to get gradients it joins with a fresh state."""
+    from fairscale_amd import _rows
+
+    if not use_helper:
+        monkeypatch.setattr(_rows, "native", None)
+    Adam, _, _ = api
+    params = _random_problem("FULL_PRECISION", cuda_device, sizes=(500, 3000, 70001), seed=13)
+    twin = [p.detach().clone().requires_grad_() for p in params]
+    opt, ref = Adam(params, lr=1e-2), Adam([twin[0], twin[2]], lr=1e-2)
+    grads = [torch.randn_like(p) * 1e-3 for p in params]
+    frozen = params[1].detach().clone()
+    for step in range(1, 6):
+        for p, q, g in zip(params, twin, grads):
+            p.grad, q.grad = g, g
+        params[1].grad = None
+        opt.step()
+        ref.step()
+    assert torch.equal(params[1], frozen) and len(opt.state[params[1]]) == 0
+    assert torch.equal(params[0], twin[0]) and torch.equal(params[2], twin[2])
+    assert next(iter(opt._plans.values())).info()["uploads"] == 1
+    params[1].grad = grads[1]
+    opt.step()
+    assert opt.state[params[1]]["step"] == 1 and opt.state[params[0]]["step"] == 6
+    assert not torch.equal(params[1], frozen)

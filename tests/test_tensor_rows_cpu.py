@@ -224,3 +224,29 @@ def test_fill_grad_rows():
     assert native.fill_grad_rows(grads, F16, -1, rows.ctypes.data)[:3] == (native.SPARSE, 3, 2)
     assert native.fill_grad_rows(grads[:2], F16, 0, rows.ctypes.data)[:3] == (native.NOT_CUDA, 3, 0)
     assert native.fill_grad_rows([], F16, -1, rows.ctypes.data)[0] == native.LENGTH
+
+
+def test_gather_with_parameters_that_sit_out():
+    """A state of None marks a parameter that had no gradient when the lists were collected: it must still
+    have none; rows are written for the others only."""
+    g = Group([7, 1, 300, 12])
+    g.params[1].grad = None
+    g.states[1] = None
+    g.rows = np.zeros((3, 6), np.int64)
+    assert g.gather() == (native.CHANGED, -1, -1, 4)
+    active = [0, 2, 3]
+    assert g.rows[:, 0].tolist() == [g.params[t].data_ptr() for t in active]
+    assert g.rows[:, 3].tolist() == [g.params[t].grad.data_ptr() for t in active]
+    assert g.rows[:, 5].tolist() == [7, 300, 12]
+    assert [s["step"] if s else None for s in g.states] == [4, None, 4, 4]
+    assert g.gather()[0] == native.UNCHANGED
+    g.params[1].grad = torch.zeros(1)  # it takes part from now on: the lists must be collected again
+    assert g.gather()[:3] == (native.STALE, 3, 1)
+    assert [s["step"] if s else None for s in g.states] == [5, None, 5, 5]
+    g.params[1].grad = None
+    g.params[3].grad = None  # one that used to take part lost its gradient
+    assert g.gather()[:3] == (native.NO_GRAD, 3, 3)
+    for t in (0, 2, 3):
+        g.states[t] = None
+        g.params[t].grad = None
+    assert g.gather()[0] == native.NO_GRAD  # nobody takes part
