@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[3], the one the metric is quoted on): a single rank's OSS shard of a
+Workload (the configuration the headline metric is quoted on): a single rank's OSS shard of a
 13B model -- one contiguous buffer of 1.63e9 parameters, MEMORY_EFFICIENT_MIXED_PRECISION (fp16
 params and grads, fp32 m/v, grads scaled by 1024).  A "step" is one ``Adam.step()`` over that shard
 with everything resident in HBM.  Prints ONE JSON line; under "also": the same number of parameters

@@ -418,7 +418,7 @@ def test_c_and_numpy_restatements_agree_bitwise(oracle, mode, eps_mode, decay):
 
 
 def test_c1_config_runs_and_descends(oracle):
-    """BASELINE config 1 (the CPU-runnable one): 2^20 fp32 params ~N(0,0.02), grads ~N(0,1e-3), 10 steps.
+    """The CPU-runnable benchmark configuration: 2^20 fp32 params ~N(0,0.02), grads ~N(0,1e-3), 10 steps.
     Every step moves every parameter by at most lr*(1+tiny) and m, v follow the exponential averages."""
     t = C.Tensors(FULL, [1 << 20], 1000)
     p0 = t.p[0].copy()

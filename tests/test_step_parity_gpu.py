@@ -108,7 +108,7 @@ DEFAULT = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, eps_mode=1, bias_corre
 
 
 def test_c1_full_precision_flat_2pow20(oracle, cuda_device):
-    """BASELINE config 1 on the GPU: one fp32 tensor of 2^20, 10 steps, fresh grads per step."""
+    """The CPU-runnable benchmark configuration on the GPU: one fp32 tensor of 2^20, 10 steps, fresh grads per step."""
     run_case(oracle, cuda_device, FULL, [1 << 20], 10, 1000, DEFAULT)
 
 
@@ -333,7 +333,7 @@ def test_nine_thousand_tiny_tensors(oracle, cuda_device):
 
 
 def test_c3_ragged_4096_tensors(oracle, cuda_device):
-    """BASELINE config 3 shape (4096 fp32 tensors, log-uniform sizes up to 2^20, wd 0.01, eps inside
+    """The ragged-list benchmark configuration (4096 fp32 tensors, log-uniform sizes up to 2^20, wd 0.01, eps inside
     the square root) at full size for 2 steps."""
     sizes = C.ragged_sizes(4096, 3000, 20.0)
     assert sum(1 for n in sizes if n % 4) > 2000
@@ -347,7 +347,7 @@ def test_c3_ragged_20_steps_smaller(oracle, cuda_device):
 
 
 def test_c2_gpt2_small_mixed_precision(oracle, cuda_device):
-    """BASELINE config 2 at full size: 148 tensors / 124M parameters, fp32 master + fp16 grads scaled by
+    """The GPT-2-small benchmark configuration at full size: 148 tensors / 124M parameters, fp32 master + fp16 grads scaled by
     65536 (passed as grad_scale) + fp16 copy-out.  Also checks p16 == half(p32) bitwise on the device."""
     sizes = [C.numel(s) for s in C.gpt2_small_shapes()]
     assert len(sizes) == 148 and sum(sizes) == 124_439_808
@@ -506,7 +506,7 @@ def _windows(n, count, width, seed):
 
 
 def test_c4_flat_shard_1p63e9_memory_efficient(oracle, cuda_device):
-    """BASELINE config 4 at its real size: one contiguous 1.63e9-element buffer, fp16 params and grads
+    """The headline benchmark configuration at its real size: one contiguous 1.63e9-element buffer, fp16 params and grads
     (grads scaled by 1024), fp32 m/v.  Data is generated on the device; the oracle re-computes the
     first/last 2*65536 elements and 48 random 65536-element windows from the pre-step state.  Also a
     misaligned sub-view is stepped and checked the same way."""
@@ -568,7 +568,7 @@ def test_single_tensor_beyond_2_to_31_elements(oracle, cuda_device):
 
 
 def test_c5_llama7b_pure_fp16_with_overflow_injection(oracle, cuda_device):
-    """BASELINE config 5 at its real size: 291 tensors / 6.74e9 fp16 parameters, fp16 grads and state
+    """The Llama-7B benchmark configuration at its real size: 291 tensors / 6.74e9 fp16 parameters, fp16 grads and state
     with optimizer-state scaling.  Step 1 is clean; in step 2 one gradient element in 10^6 is set to
     6e4, which must raise the flag.  Windows of several tensors are re-computed by the oracle."""
     from fairscale_amd import fused_adam_hip
