@@ -304,6 +304,46 @@ def test_pointer_changes_while_earlier_steps_are_in_flight(oracle, cuda_device):
     plan.close()
 
 
+def test_two_host_threads_step_their_own_lists(oracle, cuda_device):
+    """``fsadam_step`` from two threads at once (ctypes releases the interpreter lock during the call), each
+    on its own stream with its own list: the shared table cache is locked inside the library, errors are
+    kept per thread."""
+    import threading
+
+    from fairscale_amd import fused_adam_hip
+
+    cases = []
+    for k, mode in enumerate((FULL, MEMEFF)):
+        host = C.Tensors(mode, [33 + k, 5000 + k, 200000 + k], 5400 + k)
+        cases.append((host, GpuList(host, cuda_device), torch.cuda.Stream(device=cuda_device)))
+    all_grads = [[host.grads(step) for step in range(1, 9)] for host, _, _ in cases]
+    on_device = [[to_gpu(g, cuda_device) for g in per_case] for per_case in all_grads]
+    torch.cuda.synchronize(cuda_device)
+    failures = []
+
+    def worker(k):
+        try:
+            host, dev, stream = cases[k]
+            with torch.cuda.device(cuda_device), torch.cuda.stream(stream):
+                for step, g in enumerate(on_device[k], start=1):
+                    fused_adam_hip.adam(0, None, [dev.p, dev.m, dev.v, g], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, dev.found_inf, step, 1, 1, 0.0)
+        except Exception as exc:  # surfaces in the main thread below
+            failures.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize(cuda_device)
+    assert not failures, failures
+    for k, (host, dev, _) in enumerate(cases):
+        flag = np.zeros(1, np.float32)
+        for step, grads in enumerate(all_grads[k], start=1):
+            oracle_step(oracle, host, grads, flag, **dict(DEFAULT, step=step, grad_scale=1.0, optim_scale=1.0))
+        compare(host, dev, f"thread {k}")
+
+
 def test_more_lists_than_the_table_cache_holds(oracle, cuda_device):
     """``adam`` keeps the device tables of the last few lists it saw.  Twelve lists stepped in turn, three
     rounds, two modes: tables are evicted and rebuilt all the time, results stay those of the oracle."""
