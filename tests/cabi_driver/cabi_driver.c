@@ -4,7 +4,8 @@
  * three times through fsadam_step (the drop-in for fairscale.fused_adam_cuda.adam,
  * fairscale/clib/fused_adam_cuda/fused_adam_cuda.cpp:4-8) and once more through a plan; the results
  * are compared bit for bit with the CPU oracle (test infrastructure, oracle/adam_oracle.c) linked
- * into this program.  Prints one line per mode and exits 0 when everything is identical.
+ * into this program.  The gradient pass runs on values whose norms are known in closed form.
+ * Prints one line per case and exits 0 when everything is as expected.
  *
  * Built by tests/cabi_driver/Makefile (hipcc as the C compiler driver for the runtime's include and
  * library paths); run by tests/test_cabi_driver_gpu.py.
@@ -153,6 +154,70 @@ static int run_mode(int mode, const char* name) {
     return (different == 0 && h_flag == oracle_flag) ? 0 : 1;
 }
 
+/* The gradient pass on values whose norms are known in closed form: g[i] = (i % 7) - 3 as fp16, unscaled by
+ * 1/2: stored values (i % 7 - 3) / 2, sum of squares = sum over residues / 4, largest magnitude 1.5; then
+ * with one infinity planted. */
+static int run_grad_pass(void) {
+    enum { N0 = 70001, N1 = 300007 };
+    const int64_t sizes[2] = {N0, N1};
+    uint16_t* h[2];
+    void* d[2];
+    FsGradTensor rows[2];
+    double want_sum = 0.0;
+    hipStream_t stream;
+    CHECK_HIP(hipStreamCreate(&stream));
+    for (int t = 0; t < 2; ++t) {
+        h[t] = (uint16_t*)malloc((size_t)sizes[t] * 2);
+        for (int64_t i = 0; i < sizes[t]; ++i) {
+            const float v = (float)((i + t) % 7) - 3.0f;
+            h[t][i] = oracle_float_to_half(v);
+            want_sum += (double)(v * 0.5f) * (double)(v * 0.5f);
+        }
+        CHECK_HIP(hipMalloc(&d[t], (size_t)sizes[t] * 2));
+        CHECK_HIP(hipMemcpy(d[t], h[t], (size_t)sizes[t] * 2, hipMemcpyHostToDevice));
+        rows[t].g = d[t];
+        rows[t].numel = sizes[t];
+    }
+    float *d_flag, *d_max, flag = -1.f, amax = -1.f;
+    double *d_sum, sum = -1.0;
+    CHECK_HIP(hipMalloc((void**)&d_flag, 4));
+    CHECK_HIP(hipMalloc((void**)&d_max, 4));
+    CHECK_HIP(hipMalloc((void**)&d_sum, 8));
+    CHECK_HIP(hipMemset(d_flag, 0, 4));
+    int bad = 0;
+    /* read-only, then with the unscaled values written back */
+    for (int write_back = 0; write_back < 2; ++write_back) {
+        CHECK_FS(fsadam_grad_pass(rows, 2, FSADAM_GRAD_F16, 0.5f, NULL, write_back, d_flag, d_sum, d_max, stream));
+        CHECK_HIP(hipStreamSynchronize(stream));
+        CHECK_HIP(hipMemcpy(&flag, d_flag, 4, hipMemcpyDeviceToHost));
+        CHECK_HIP(hipMemcpy(&amax, d_max, 4, hipMemcpyDeviceToHost));
+        CHECK_HIP(hipMemcpy(&sum, d_sum, 8, hipMemcpyDeviceToHost));
+        const int ok = flag == 0.0f && amax == 1.5f && sum == want_sum; /* quarters and small integers: exact in float32 and float64 */
+        printf("gradient pass, write_back %d: flag %g, max %g, sum of squares %.17g (expected %.17g) %s\n", write_back, flag, amax, sum,
+               want_sum, ok ? "ok" : "WRONG");
+        bad |= !ok;
+    }
+    uint16_t first = 0;
+    CHECK_HIP(hipMemcpy(&first, (char*)d[0] + 2 * 6, 2, hipMemcpyDeviceToHost)); /* element 6 was +3, now +1.5 */
+    bad |= first != oracle_float_to_half(1.5f);
+    const uint16_t inf = 0x7c00;
+    CHECK_HIP(hipMemcpy((char*)d[1] + 2 * 12345, &inf, 2, hipMemcpyHostToDevice));
+    CHECK_FS(fsadam_grad_pass(rows, 2, FSADAM_GRAD_F16, 1.0f, NULL, 0, d_flag, d_sum, d_max, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    CHECK_HIP(hipMemcpy(&flag, d_flag, 4, hipMemcpyDeviceToHost));
+    printf("gradient pass with an infinity planted: flag %g %s\n", flag, flag == 1.0f ? "ok" : "WRONG");
+    bad |= flag != 1.0f;
+    for (int t = 0; t < 2; ++t) {
+        CHECK_HIP(hipFree(d[t]));
+        free(h[t]);
+    }
+    CHECK_HIP(hipFree(d_flag));
+    CHECK_HIP(hipFree(d_max));
+    CHECK_HIP(hipFree(d_sum));
+    CHECK_HIP(hipStreamDestroy(stream));
+    return bad;
+}
+
 int main(void) {
     int n_dev = 0;
     if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev < 1) {
@@ -166,6 +231,7 @@ int main(void) {
     bad |= run_mode(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION, "MEMORY_EFFICIENT_MIXED_PRECISION");
     bad |= run_mode(FSADAM_PURE_FP16, "PURE_FP16");
     bad |= run_mode(FSADAM_FULL_PRECISION_FP16_COPY, "FULL_PRECISION_FP16_COPY");
+    bad |= run_grad_pass();
     if (fsadam_clear_cache() != FSADAM_OK) bad |= 1;
     printf(bad ? "FAILED\n" : "all modes bit-identical to the oracle\n");
     return bad;

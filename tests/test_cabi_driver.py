@@ -36,3 +36,4 @@ def test_every_mode_matches_the_oracle_from_plain_c(cuda_device):
     assert proc.returncode == 0, proc.stdout
     assert "all modes bit-identical to the oracle" in proc.stdout
     assert proc.stdout.count(" 0 differ") == 5
+    assert proc.stdout.count("ok") >= 3 and "WRONG" not in proc.stdout  # the gradient pass lines
