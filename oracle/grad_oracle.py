@@ -8,8 +8,9 @@ Restates, over numpy arrays, what the reference's callers compute on the gradien
 * ``calc_grad_norm`` (``fairscale/internal/params.py:59-76``): the 2-norm and the max-norm of all
   gradients as one vector, "in full precision no matter what".
 
-Sums are taken in float64 here, so the oracle is the exact value the device result is compared with
-under a tolerance (the device squares in float32 and then sums in float64).  Pinned in
+Squares are taken in float32, as ``torch.norm(..., dtype=torch.float32)`` takes them (a gradient above
+1.8e19 squares to infinity there, and the norm is infinite), and summed in float64: up to the order
+of the additions this is the value the device result is compared with under a tolerance.  Pinned in
 ``tests/test_grad_pass_cpu.py`` against torch's own CPU implementation of the unscale op and
 ``torch.norm``.
 """
@@ -37,7 +38,7 @@ def grad_pass_numpy(grads: Sequence[np.ndarray], inv_scale: float, write_back: b
         with np.errstate(all="ignore"):
             r = g if inv == np.float32(1.0) else (f * inv).astype(g.dtype)
             u = r.astype(np.float32)
-            total += float((u.astype(np.float64) ** 2).sum())
+            total += float((u * u).astype(np.float64).sum())  # float32 squares, float64 sum
             m = np.abs(u).max()  # numpy's max propagates NaN
         abs_max = m if (np.isnan(m) or m > abs_max) and not np.isnan(abs_max) else abs_max
         if write_back and r is not g:

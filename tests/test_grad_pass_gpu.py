@@ -1,9 +1,9 @@
 """GPU parity of the fused gradient pass (``fsadam_grad_pass`` through the C ABI) against its oracle.
 
 Bars: what is stored (unscaled gradients) and the overflow flag are bit-exact; the max norm is exact
-(a maximum does not round); the sum of squares is within 1e-6 relative of the float64 oracle (the
-device squares in float32, like ``torch.norm(..., dtype=float32)``, and then adds in float64 in a fixed
-order) and bit-identical between runs."""
+(a maximum does not round); the sum of squares is within 1e-6 relative of the oracle (both square in
+float32, like ``torch.norm(..., dtype=float32)``, and add in float64; the device in a fixed order of its
+own) and bit-identical between runs; where a float32 square overflows both are infinite."""
 from __future__ import annotations
 
 import math
@@ -62,7 +62,7 @@ def check(host, dev, stats, want, what):
         assert got_mx == mx, what
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(50))
 def test_random_gradient_lists_match_the_oracle(cuda_device, seed):
     """Drawn configurations: dtype, list, sizes around the tile sizes of both kinds of pass, an element
     offset per tensor, factors that are 1, a power of two, a half, not a half, tiny and huge, with and
