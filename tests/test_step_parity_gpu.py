@@ -362,6 +362,49 @@ def test_more_lists_than_the_table_cache_holds(oracle, cuda_device):
         compare(host, dev, f"list {k}")
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_extreme_states_and_hyperparameters_match_the_oracle(oracle, cuda_device, seed):
+    """Drawn once more, now from the edges: infinities, NaNs, the largest and smallest magnitudes, zeros of both
+    signs and a negative second moment planted in p, m and v before the first step; lr from 1e-8 to 1,
+    betas 0 / 0.5 / 0.999, eps 0 or 1, decay up to 10, scales from 1e-3 to 2^18 (PURE_FP16 optimizer
+    scales from 1/8 to 2^16), a step number of 100000.  IEEE arithmetic decides every result, on both
+    sides the same."""
+    import random
+
+    rng = random.Random(20000 + seed)
+    mode = rng.choice([FULL, MIXED, MEMEFF, PURE16])
+    tile = 512 if mode == PURE16 else 256
+    sizes = [rng.choice([1, 3, tile - 1, tile, tile + 1, 5 * tile + 3, 40000, 131072, 140001]) for _ in range(rng.randrange(1, 8))]
+    host = C.Tensors(mode, sizes, 21000 + seed)
+    with np.errstate(over="ignore"):
+        for arrs in (host.p, host.m, host.v):
+            for a in arrs:
+                info = np.finfo(a.dtype)
+                for value in (np.inf, -np.inf, np.nan, info.max, -info.max, info.tiny, info.smallest_subnormal, -info.smallest_subnormal,
+                              0.0, -0.0, 1.0, -1e-30 if a.dtype == np.float32 else -6e-8):
+                    if rng.random() < 0.25:
+                        a[rng.randrange(a.size)] = value
+        if mode == MIXED:
+            host.p16 = [x.astype(np.float16) for x in host.p]
+    misalign = {name: [rng.choice([0, 0, 1, 3]) for _ in sizes] for name in ("p", "m", "v", "g", "p16")}
+    dev = GpuList(host, cuda_device, misalign)
+    hyper = dict(lr=rng.choice([1e-3, 1.0, 1e-8]), beta1=rng.choice([0.9, 0.0, 0.999]), beta2=rng.choice([0.999, 0.5, 0.0]),
+                 eps=rng.choice([1e-8, 0.0, 1.0]), eps_mode=rng.randrange(2), bias_correction=rng.randrange(2),
+                 decay=rng.choice([0.0, 0.01, 10.0]))
+    grad_scale = rng.choice([1.0, 128.0, 3.0, 1e-3, 65536.0 * 4])
+    optim_scale = rng.choice([65536.0, 1.0, 1000.0, 2.0 ** -3]) if mode == PURE16 else 1.0
+    flag = np.zeros(1, np.float32)
+    print(f"seed {seed}: mode {mode}, sizes {sizes}, {hyper}, grad_scale {grad_scale}, optim_scale {optim_scale}", flush=True)
+    for step in (1, 2, 3):
+        with np.errstate(over="ignore"):
+            grads = host.grads(step, g_std=rng.choice([1e-3, 1.0, 1e-6]), scale=grad_scale)
+        kw = dict(hyper, step=step if rng.random() < 0.8 else 100000, grad_scale=grad_scale, optim_scale=optim_scale)
+        dev.step(grads, **kw)
+        oracle_step(oracle, host, grads, flag, **kw)
+        compare(host, dev, f"seed {seed} mode {mode} step {step}")
+    assert float(dev.found_inf.item()) == float(flag[0])
+
+
 def test_zero_sized_tensors_in_list(oracle, cuda_device):
     run_case(oracle, cuda_device, FULL, [0, 5, 0, 0, 20000, 0], 2, 4300, DEFAULT)
 
