@@ -662,3 +662,48 @@ def test_frozen_parameters_do_not_disable_the_steady_state_walk(api, cuda_device
     opt.step()
     assert opt.state[params[1]]["step"] == 1 and opt.state[params[0]]["step"] == 6
     assert not torch.equal(params[1], frozen)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_drawn_list_defects_are_refused_by_both_walks(cuda_device, seed, monkeypatch):
+    """One defect planted at a drawn place of a drawn list (stride, dtype, numel, a host tensor, a missing entry,
+    a sparse tensor): ``adam`` raises ``RuntimeError`` with the C++ helper and without it, and the same list
+    without the defect goes through."""
+    import random
+
+    from fairscale_amd import _rows, fused_adam_hip
+
+    rng = random.Random(31000 + seed)
+    mode_name = rng.choice(["FULL", "MIXED", "MEMEFF", "PURE16"])
+    dts = {"FULL": (torch.float32,) * 4, "MIXED": (torch.float32, torch.float32, torch.float32, torch.float16, torch.float16),
+           "MEMEFF": (torch.float16, torch.float32, torch.float32, torch.float16), "PURE16": (torch.float16,) * 4}[mode_name]
+    sizes = [rng.choice([1, 5, 300, 4097]) for _ in range(rng.randrange(1, 6))]
+    make = lambda: [[torch.zeros(n, dtype=dt, device=cuda_device) for n in sizes] for dt in dts]  # noqa: E731
+    flag = torch.zeros(1, device=cuda_device)
+    call = lambda lists: fused_adam_hip.adam(0, None, lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 65536.0 if mode_name == "PURE16" else 1.0,  # noqa: E731
+                                             flag, 1, 1, 1, 0.0)
+    d, t = rng.randrange(len(dts)), rng.randrange(len(sizes))
+    n, dt = sizes[t], dts[d]
+    defect = rng.choice(["stride", "dtype", "numel", "host", "length", "sparse"])
+    if defect == "stride" and n == 1:
+        defect = "numel"  # a one-element tensor is contiguous whatever its stride
+    for use_helper in (True, False):
+        if not use_helper:
+            monkeypatch.setattr(_rows, "native", None)
+        call(make())
+        lists = make()
+        if defect == "stride":
+            lists[d][t] = torch.zeros(2 * n, dtype=dt, device=cuda_device)[::2]
+        elif defect == "dtype":
+            lists[d][t] = torch.zeros(n, dtype=torch.float64, device=cuda_device)
+        elif defect == "numel":
+            lists[d][t] = torch.zeros(n + 1, dtype=dt, device=cuda_device)
+        elif defect == "host":
+            lists[d][t] = torch.zeros(n, dtype=dt)
+        elif defect == "length":
+            lists[d] = lists[d][:-1] if d > 0 else lists[d] + [torch.zeros(3, dtype=dt, device=cuda_device)]
+        else:
+            lists[d][t] = torch.zeros(n, dtype=dt, device=cuda_device).to_sparse()
+        with pytest.raises((RuntimeError, NotImplementedError)):
+            call(lists)
+    torch.cuda.synchronize(cuda_device)
