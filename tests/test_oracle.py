@@ -504,3 +504,60 @@ def test_torch_cpu_baseline_matches_oracle(oracle, mode):
         else:
             ok = diff <= 1e-5 * np.abs(want) + 1e-5 * scale
         assert ok.all()
+
+
+# ---- what the stated tolerance is for: the reference's own build flags
+
+def _fast_math_step(O, p, m, v, g, *, lr, beta1, beta2, eps, step, rng, ulps=2):
+    """FULL_PRECISION step as nvcc's ``--use_fast_math`` (setup.py:50) is allowed to evaluate it:
+    multiply-adds fused (one rounding), division and square root off by up to ``ulps`` units in the last
+    place in a drawn direction, denormal inputs and results flushed to zero.  Same equations,
+    fused_adam_cuda_kernel.cu:115-130, step size as :153-162."""
+    f, d = np.float32, np.float64
+
+    def ftz(x):
+        return np.where(np.abs(x) < np.finfo(f).tiny, f(0), x).astype(f)
+
+    def wobble(x):
+        bits = x.view(np.int32) + rng.integers(-ulps, ulps + 1, size=x.shape).astype(np.int32)
+        return np.where(np.isfinite(x) & (x != 0), bits.view(f), x).astype(f)
+
+    b1, b2, e = f(beta1), f(beta2), f(eps)
+    ss = O.step_size_numpy(lr, beta1, beta2, step, 1)
+    g, m_in, v_in, p_in = ftz(g), ftz(m), ftz(v), ftz(p)
+    mom = ftz((d(b1) * d(m_in) + d(f(1) - b1) * d(g)).astype(f))                      # fma(b1, m, (1-b1)*g): one rounding
+    vel = ftz((d(b2) * d(v_in) + d(((f(1) - b2) * g).astype(f)) * d(g)).astype(f))   # fma((1-b2)*g, g, b2*v)
+    denom = ftz(wobble(np.sqrt(vel)) + e)
+    update = ftz(wobble((mom / denom).astype(f)))
+    new_p = ftz((d(p_in) - d(ss) * d(update)).astype(f))                              # fma(-step_size, update, p)
+    p[...], m[...], v[...] = new_p, mom, vel
+
+
+def test_fast_math_reading_of_the_reference_stays_inside_the_tolerance(oracle):
+    """The oracle is the IEEE reading of the reference source; the reference binary was built with
+    ``--use_fast_math``.  Ten steps of the CPU-runnable configuration evaluated both ways stay within
+    1e-6 of (the element's magnitude + the stream's root mean square) in p, m and v: that is what the
+    1e-6 bar can absorb of what cannot be pinned without the binary.  Measured against each element's OWN magnitude
+    the two readings are further apart for the few per cent of elements that lie near zero (an error of
+    two units in the last place of the update is 2e-10, which is 2e-6 of a parameter of 1e-4): no
+    implementation could match the binary more closely there, and the GPU is compared with the IEEE
+    oracle bit for bit instead."""
+    O = oracle
+    n = 1 << 16
+    rng = np.random.default_rng(1000)
+    p0 = (rng.standard_normal(n).astype(np.float32) * np.float32(0.02))
+    ieee = [p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)]
+    fast = [p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)]
+    for step in range(1, 11):
+        g = rng.standard_normal(n).astype(np.float32) * np.float32(1e-3)
+        O.step_c(O.FULL_PRECISION, ieee[0], ieee[1], ieee[2], g, None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=step)
+        _fast_math_step(O, fast[0], fast[1], fast[2], g.copy(), lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=step, rng=rng)
+        for name, a, b in zip("pmv", ieee, fast):
+            err = np.abs(a.astype(np.float64) - b)
+            rms = math.sqrt(float((a.astype(np.float64) ** 2).mean()))
+            gate = 1e-6 * (np.abs(a) + rms)
+            assert (err <= gate).all(), f"step {step} {name}: worst {float((err / gate).max()):.2f} times the gate"
+    differing = sum(int((a != b).sum()) for a, b in zip(ieee, fast))
+    assert differing > n  # the two readings do differ in the last places: the comparison is not vacuous
+    own = np.abs(ieee[0].astype(np.float64) - fast[0]) / np.maximum(np.abs(ieee[0]), 1e-30)
+    assert 0.001 < float((own > 1e-6).mean()) < 0.05  # near-zero parameters: beyond 1e-6 of their own magnitude
