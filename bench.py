@@ -106,10 +106,12 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
     return out
 
 
-def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000):
+def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=False):
     """4096 fp32 tensors of log-uniform sizes (numel = max(1, round(2**U(0, 20)))), FULL_PRECISION with weight
     decay and eps inside the square root: the list-handling case.  Host time per step (the calls return
-    without waiting), device time per step, and wall time of back-to-back steps."""
+    without waiting), device time per step, and wall time of back-to-back steps.  ``packed``: the
+    parameters are views laid back to back into one flat buffer that starts one element in (so nearly every
+    tensor starts between cache lines), the gradients likewise."""
     import random
 
     from fairscale_amd import _rows
@@ -117,9 +119,18 @@ def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000):
 
     rng = random.Random(seed)
     sizes = [max(1, round(2 ** rng.uniform(0.0, 20.0))) for _ in range(count)]
-    params = [torch.empty(n, device=device).normal_(0, 0.02).requires_grad_() for n in sizes]
-    for p in params:
-        p.grad = torch.empty_like(p).normal_(0, 1e-3)
+    if packed:
+        flat = torch.empty(sum(sizes) + 1, device=device).normal_(0, 0.02)
+        flat_grad = torch.empty_like(flat).normal_(0, 1e-3)
+        params, at = [], 1
+        for n in sizes:
+            params.append(flat[at:at + n].requires_grad_())
+            params[-1].grad = flat_grad[at:at + n]
+            at += n
+    else:
+        params = [torch.empty(n, device=device).normal_(0, 0.02).requires_grad_() for n in sizes]
+        for p in params:
+            p.grad = torch.empty_like(p).normal_(0, 1e-3)
     opt = Adam(params, lr=1e-3, weight_decay=0.01, eps_inside_sqrt=True, precision=Precision.FULL_PRECISION)
     for _ in range(warmup):
         opt.step()
@@ -252,6 +263,7 @@ def main():
     if not args.no_also:
         also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
         also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device)
+        also["ragged_4096_packed_views_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device, packed=True)
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"

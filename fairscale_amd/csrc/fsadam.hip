@@ -82,6 +82,7 @@ struct Options {
     int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
     int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
     int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
+    int64_t align_heads = 1;        // 1: a tensor whose streams start off a cache line gives up a short head so that the rest starts on one
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -138,11 +139,55 @@ int validate_rows(const FsAdamTensor* tensors, int64_t n, int mode) {
     return FSADAM_OK;
 }
 
-// Every stream aligned to the kElems elements a lane moves per instruction: the tensor runs at full speed.
-bool row_vector_ok(const FsAdamTensor& r, int mode) {
+char* advance(const void* base, int64_t elems, int elem_size) {
+    return const_cast<char*>(static_cast<const char*>(base)) + elems * elem_size;
+}
+
+// Every stream, `first` elements in, aligned to the kElems elements a lane moves per instruction.
+bool row_vector_ok(const FsAdamTensor& r, int mode, int64_t first = 0) {
     const uintptr_t e = mode_elems(mode);
-    return aligned_to(r.p, e * size_p(mode)) && aligned_to(r.m, e * size_s(mode)) && aligned_to(r.v, e * size_s(mode)) &&
-           aligned_to(r.g, e * size_g(mode)) && (!mode_has_copy(mode) || aligned_to(r.p_copy, e * 2));
+    return aligned_to(advance(r.p, first, size_p(mode)), e * size_p(mode)) && aligned_to(advance(r.m, first, size_s(mode)), e * size_s(mode)) &&
+           aligned_to(advance(r.v, first, size_s(mode)), e * size_s(mode)) && aligned_to(advance(r.g, first, size_g(mode)), e * size_g(mode)) &&
+           (!mode_has_copy(mode) || aligned_to(advance(r.p_copy, first, 2), e * 2));
+}
+
+// Where a tensor's streams start relative to cache lines decides how fast its tiles run: a wave moves
+// 512 or 1024 contiguous bytes of a stream per instruction, and when those spans straddle 128-byte
+// lines every line is touched by two instructions (partial-line writes, reads fetched twice): a list of
+// views packed back to back measured 62-65 % of the HBM rate against 77-79 % for the same list on
+// line boundaries.  A view cannot be moved, but its first few elements can be given to a short
+// descriptor of their own, so that all the tiles behind it start where the streams are aligned.
+// The head is chosen among the counts that bring one of the streams onto a 128-byte or 1024-byte
+// boundary, by the bytes each stream moves per element times how far off it stays:
+// nothing for a 1 KiB boundary, a little for a line boundary, most for anything else.
+constexpr int64_t kHeadMinElems = 8192;  // shorter tensors are left alone: a head would add a workgroup to a handful
+int64_t misalignment_cost(const void* ptr, int64_t first, int elem_size, int bytes_moved) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(advance(ptr, first, elem_size));
+    const int64_t off = (a & 1023u) == 0 ? 0 : (a & 127u) == 0 ? 1 : (a & 15u) == 0 ? 5 : 6;
+    return off * bytes_moved;
+}
+int64_t head_elems(const FsAdamTensor& r, int mode, const Options& opt) {
+    if (!opt.align_heads || r.numel < kHeadMinElems) return 0;
+    struct Stream { const void* ptr; int size, moved; };
+    const Stream streams[5] = {{r.p, size_p(mode), 2 * size_p(mode)}, {r.m, size_s(mode), 2 * size_s(mode)}, {r.v, size_s(mode), 2 * size_s(mode)},
+                               {r.g, size_g(mode), size_g(mode)}, {mode_has_copy(mode) ? r.p_copy : nullptr, 2, 2}};
+    auto cost = [&](int64_t head) {
+        int64_t c = 0;
+        for (const Stream& st : streams)
+            if (st.ptr) c += misalignment_cost(st.ptr, head, st.size, st.moved);
+        return c;
+    };
+    int64_t best = 0, best_cost = cost(0);
+    for (const Stream& st : streams) {
+        if (!st.ptr) continue;
+        for (uintptr_t boundary : {uintptr_t(128), uintptr_t(1024)}) {
+            const uintptr_t a = reinterpret_cast<uintptr_t>(st.ptr);
+            const int64_t head = (int64_t)(((boundary - (a & (boundary - 1))) & (boundary - 1)) / st.size);
+            const int64_t c = cost(head);
+            if (c < best_cost || (c == best_cost && head < best)) { best = head; best_cost = c; }
+        }
+    }
+    return best;
 }
 
 int64_t floor_pow2(int64_t x) {
@@ -176,10 +221,11 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
         const int64_t numel = tensors[t].numel;
         L.total_elems += numel;
         if (numel == 0) { L.n_empty += 1; continue; }
-        (row_vector_ok(tensors[t], mode) ? L.n_vector : L.n_scalar) += 1;
-        if (numel >= kLargeThreshold) {
+        const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
+        (row_vector_ok(tensors[t], mode, head) ? L.n_vector : L.n_scalar) += 1;
+        if (body >= kLargeThreshold) {
             L.n_large += 1;
-            if (min_large == 0 || numel < min_large) min_large = numel;
+            if (min_large == 0 || body < min_large) min_large = body;
         } else {
             L.n_small += 1;
         }
@@ -189,8 +235,10 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = tensors[t].numel;
         if (numel == 0) continue;
-        if (numel >= kLargeThreshold) L.n_large_descs += ceil_div(numel, L.large_chunk_elems);
-        else L.n_small_descs += ceil_div(numel, L.tile_elems);
+        const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
+        L.n_small_descs += ceil_div(head, L.tile_elems);
+        if (body >= kLargeThreshold) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        else L.n_small_descs += ceil_div(body, L.tile_elems);
     }
     return L;
 }
@@ -262,24 +310,22 @@ void plan_release_buffers(FsAdamPlan* plan) {
     plan->current = -1;
 }
 
-char* advance(const void* base, int64_t elems, int elem_size) {
-    return const_cast<char*>(static_cast<const char*>(base)) + elems * elem_size;
-}
-
-void fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t chunk_elems, bool vec) {
-    const int64_t chunks = ceil_div(r.numel, chunk_elems);
+// Descriptors for elements [start, start + count) of a tensor, chunk_elems each; returns how many.
+int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t start, int64_t count, int64_t chunk_elems, bool vec) {
+    const int64_t chunks = ceil_div(count, chunk_elems);
     for (int64_t c = 0; c < chunks; ++c) {
-        const int64_t first = c * chunk_elems;
+        const int64_t first = start + c * chunk_elems;
         ChunkDesc& d = out[c];
         d.p = advance(r.p, first, size_p(mode));
         d.m = advance(r.m, first, size_s(mode));
         d.v = advance(r.v, first, size_s(mode));
         d.g = advance(r.g, first, size_g(mode));
         d.p_copy = mode_has_copy(mode) ? advance(r.p_copy, first, 2) : nullptr;
-        d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - first);
+        d.n = (uint32_t)std::min<int64_t>(chunk_elems, start + count - first);
         d.vector_ok = vec ? 1u : 0u;
         d.pad = 0;
     }
+    return chunks;
 }
 
 template <int MODE, int BLOCK, int GROUPS>
@@ -371,15 +417,14 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     for (int64_t t = 0; t < n; ++t) {
         const FsAdamTensor& r = tensors[t];
         if (r.numel == 0) continue;
-        const bool vec = plan->opt.unaligned_vectors != 0 || row_vector_ok(r, plan->mode);
-        if (r.numel >= kLargeThreshold) {
-            fill_descs(large, r, plan->mode, L.large_chunk_elems, vec);
-            large += ceil_div(r.numel, L.large_chunk_elems);
-        } else {
-            fill_descs(small, r, plan->mode, L.tile_elems, vec);
-            small += ceil_div(r.numel, L.tile_elems);
-        }
+        const int64_t head = head_elems(r, plan->mode, plan->opt), body = r.numel - head;
+        const bool vec = plan->opt.unaligned_vectors != 0 || row_vector_ok(r, plan->mode, head);
+        small += fill_descs(small, r, plan->mode, 0, head, L.tile_elems, plan->opt.unaligned_vectors != 0);
+        if (body >= kLargeThreshold) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems, vec);
+        else small += fill_descs(small, r, plan->mode, head, body, L.tile_elems, vec);
     }
+    if (large != slot.h_table + L.n_large_descs || small != slot.h_table + n_descs)
+        return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(tensors, tensors + n);
     if (n_descs > 0)
@@ -437,6 +482,7 @@ struct GradPlan {
     int64_t lds_throttle = 0;
     int64_t max_large_chunk = kMaxLargeChunk;
     int64_t unaligned_vectors = 1;
+    int64_t align_heads = 1;
     int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
     std::vector<FsGradTensor> rows;
     Layout layout;
@@ -455,18 +501,28 @@ constexpr int kReduceBlocks = 512;
 int grad_elem_size(int dtype) { return dtype == FSADAM_GRAD_F16 ? 2 : 4; }
 int64_t grad_tile_elems(int dtype, int64_t items) { return 64 * (16 / grad_elem_size(dtype)) * items; }
 
-Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk) {
+// The one stream of the gradient pass: the elements in front of the next 1 KiB boundary go to a
+// descriptor of their own, as in the step.
+int64_t grad_head_elems(const FsGradTensor& r, int elem_size, int64_t align_heads) {
+    if (!align_heads || r.numel < kHeadMinElems) return 0;
+    const uintptr_t a = reinterpret_cast<uintptr_t>(r.g);
+    return (int64_t)(((1024 - (a & 1023u)) & 1023u) / (uintptr_t)elem_size);
+}
+
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk, int64_t align_heads) {
     Layout L;
     L.tile_elems = grad_tile_elems(dtype, items);
+    const int esz = grad_elem_size(dtype);
     int64_t min_large = 0;
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = grads[t].numel;
         L.total_elems += numel;
         if (numel == 0) { L.n_empty += 1; continue; }
-        (aligned_to(grads[t].g, 16) ? L.n_vector : L.n_scalar) += 1;
-        if (numel >= kLargeThreshold) {
+        const int64_t head = grad_head_elems(grads[t], esz, align_heads), body = numel - head;
+        (aligned_to(advance(grads[t].g, head, esz), 16) ? L.n_vector : L.n_scalar) += 1;
+        if (body >= kLargeThreshold) {
             L.n_large += 1;
-            if (min_large == 0 || numel < min_large) min_large = numel;
+            if (min_large == 0 || body < min_large) min_large = body;
         } else {
             L.n_small += 1;
         }
@@ -475,8 +531,10 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = grads[t].numel;
         if (numel == 0) continue;
-        if (numel >= kLargeThreshold) L.n_large_descs += ceil_div(numel, L.large_chunk_elems);
-        else L.n_small_descs += ceil_div(numel, L.tile_elems);
+        const int64_t head = grad_head_elems(grads[t], esz, align_heads), body = numel - head;
+        L.n_small_descs += ceil_div(head, L.tile_elems);
+        if (body >= kLargeThreshold) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        else L.n_small_descs += ceil_div(body, L.tile_elems);
     }
     return L;
 }
@@ -494,8 +552,10 @@ void grad_plan_free(GradPlan* plan) {
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
-void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves) {
+void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves,
+                int64_t* align_heads) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    *align_heads = g_opt.align_heads;
     // a pass that only reads pays for every small store it makes: 16 tiles share one partial
     *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
     *max_large_chunk = g_opt.max_large_chunk;
@@ -505,7 +565,7 @@ void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_ch
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
-    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk);
+    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk, plan->align_heads);
     const int64_t k = L.large_chunk_elems / L.tile_elems;
     const int64_t n_blocks = L.n_large_descs * k + L.n_small_descs;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
@@ -547,19 +607,26 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     for (int64_t t = 0; t < n; ++t) {
         const FsGradTensor& r = grads[t];
         if (r.numel == 0) continue;
-        const bool is_large = r.numel >= kLargeThreshold;
-        const int64_t chunk_elems = is_large ? L.large_chunk_elems : L.tile_elems;
-        const int64_t chunks = ceil_div(r.numel, chunk_elems);
-        ChunkDesc*& out = is_large ? large : small;
-        for (int64_t c = 0; c < chunks; ++c) {
-            ChunkDesc& d = out[c];
-            std::memset(&d, 0, sizeof(d));
-            d.g = advance(r.g, c * chunk_elems, esz);
-            d.n = (uint32_t)std::min<int64_t>(chunk_elems, r.numel - c * chunk_elems);
-            d.vector_ok = (plan->unaligned_vectors != 0 || aligned_to(r.g, 16)) ? 1u : 0u;
+        const int64_t head = grad_head_elems(r, esz, plan->align_heads);
+        // pieces: the head (tile-sized descriptors), then the rest in shared chunks or tiles
+        const struct { int64_t start, count; bool large; } pieces[2] = {{0, head, false}, {head, r.numel - head, r.numel - head >= kLargeThreshold}};
+        for (const auto& piece : pieces) {
+            const int64_t chunk_elems = piece.large ? L.large_chunk_elems : L.tile_elems;
+            const int64_t chunks = ceil_div(piece.count, chunk_elems);
+            ChunkDesc*& out = piece.large ? large : small;
+            for (int64_t c = 0; c < chunks; ++c) {
+                ChunkDesc& d = out[c];
+                std::memset(&d, 0, sizeof(d));
+                const int64_t first = piece.start + c * chunk_elems;
+                d.g = advance(r.g, first, esz);
+                d.n = (uint32_t)std::min<int64_t>(chunk_elems, piece.start + piece.count - first);
+                d.vector_ok = (plan->unaligned_vectors != 0 || aligned_to(advance(r.g, piece.start, esz), 16)) ? 1u : 0u;
+            }
+            out += chunks;
         }
-        out += chunks;
     }
+    if (large != slot.h_table + L.n_large_descs || small != slot.h_table + n_descs)
+        return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(grads, grads + n);
     if (n_descs > 0)
@@ -649,7 +716,7 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
 
 bool same_options(const Options& a, const Options& b) {
     return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap &&
-           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors;
+           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors && a.align_heads == b.align_heads;
 }
 
 }  // namespace
@@ -691,6 +758,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "unaligned_vectors") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "unaligned_vectors must be 0 or 1");
         g_opt.unaligned_vectors = value;
+    } else if (k == "align_heads") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "align_heads must be 0 or 1");
+        g_opt.align_heads = value;
     } else if (k == "max_large_chunk") {
         if (value < 4096 || value > kMaxLargeChunk || (value & (value - 1)) != 0)
             return fail(FSADAM_EINVAL, "max_large_chunk must be a power of two in [4096, 2^24] elements");
@@ -720,6 +790,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "xcd_remap") *value = g_opt.xcd_remap;
     else if (k == "max_large_chunk") *value = g_opt.max_large_chunk;
     else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
+    else if (k == "align_heads") *value = g_opt.align_heads;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else if (k == "grad_waves") *value = g_opt.grad_waves;
@@ -748,9 +819,23 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
     out->grid_large = L.n_large_descs * (L.large_chunk_elems / L.tile_elems);
     out->grid_small = L.n_small_descs;
     for (int64_t t = 0; t < n_tensors; ++t) {
-        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (tensors[t].numel >= kLargeThreshold ? 2 : 1);
-        if (vector_ok) vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode)) ? 1 : 0;
+        const int64_t head = tensors[t].numel > 0 ? head_elems(tensors[t], precision_mode, opt) : 0;
+        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (tensors[t].numel - head >= kLargeThreshold ? 2 : 1);
+        if (vector_ok) vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode, head)) ? 1 : 0;
     }
+    return FSADAM_OK;
+}
+
+int fsadam_head_elems(const FsAdamTensor* tensor, int precision_mode, int64_t* head) {
+    if (!head) return fail(FSADAM_EINVAL, "head is NULL");
+    int rc = validate_rows(tensor, 1, precision_mode);
+    if (rc) return rc;
+    Options opt;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        opt = g_opt;
+    }
+    *head = tensor->numel > 0 ? head_elems(*tensor, precision_mode, opt) : 0;
     return FSADAM_OK;
 }
 
@@ -878,15 +963,15 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves;
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads;
     grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
-               &cur_waves);
+               &cur_waves, &cur_heads);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && c->align_heads == cur_heads && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -911,6 +996,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->lds_throttle = cur_lds;
         victim->max_large_chunk = cur_chunk;
         victim->unaligned_vectors = cur_unaligned;
+        victim->align_heads = cur_heads;
         victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }

@@ -19,6 +19,9 @@ Deliberate differences, all supersets of the reference behaviour:
   round-trips them through fp16, adam.py:176-182).
 * The fp32 master copies of MIXED_PRECISION carry no ``.grad`` (the reference allocates a zero one per
   copy, adam.py:128, and never reads it).
+* ``exp_avg``/``exp_avg_sq`` of a parameter that is a view starting between 128-byte lines (packed into a
+  flat buffer) are views too, 512 elements into a slightly longer allocation at most, so that state and
+  parameter leave their lines at the same element (``zeros_like`` in the reference, adam.py:226-228).
 """
 from __future__ import annotations
 
@@ -54,6 +57,22 @@ _NATIVE_MODE = {
 }
 
 _MAX_OPTIM_SCALE = 2 ** 16
+
+
+def _state_like(p: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Zeros of ``p``'s shape for its exp_avg / exp_avg_sq.  A parameter that starts between cache lines (a
+    view packed into a flat buffer) gets state that starts as many elements past a 1 KiB boundary as the
+    parameter does, modulo 512, inside an allocation 512 elements longer: the native layout then finds ONE
+    head length that puts the parameter's and the state's tiles on line boundaries together; with state
+    on its own boundaries the parameter's stream would stay split across lines."""
+    n = p.numel()
+    if n < 8192 or p.data_ptr() % 128 == 0 or not p.is_contiguous():
+        return torch.zeros_like(p, dtype=dtype)
+    want = (p.data_ptr() // p.element_size()) % 512
+    buf = torch.zeros(n + 512, dtype=dtype, device=p.device)
+    have = (buf.data_ptr() // buf.element_size()) % 512
+    start = (want - have) % 512
+    return buf[start:start + n].view(p.shape)
 
 
 class _VersionedState(defaultdict):
@@ -274,8 +293,9 @@ class Adam(torch.optim.Optimizer):
             state = state_map[p]
             if len(state) == 0:  # adam.py:223-228
                 state["step"] = 0
-                state["exp_avg"] = torch.zeros_like(p, dtype=optim_type)
-                state["exp_avg_sq"] = torch.zeros_like(p, dtype=optim_type)
+                like = masters[pj] if mixed else p
+                state["exp_avg"] = _state_like(like, optim_type)
+                state["exp_avg_sq"] = _state_like(like, optim_type)
             step_no = state["step"] = state["step"] + 1  # the call uses the last parameter's counter (adam.py:272)
             states.append(state)
             lists = batches.get(p.device)

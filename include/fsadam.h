@@ -123,6 +123,10 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "unaligned_vectors"  1 (default): full tiles of a tensor whose streams are only element-aligned (a view that
  *                   starts at an odd element) still move with 64/128-bit vector instructions; 0: such tensors
  *                   are processed element by element (measured 1.5-2x slower)
+ *   "align_heads"   1 (default): a tensor of 8192 elements or more whose streams start off a 128-byte line (a view
+ *                   into a flat buffer) gives its first elements, at most 511, to a short descriptor of their own, so
+ *                   that every tile behind them starts on line boundaries (see fsadam_head_elems); 0: tiles start
+ *                   at element 0 wherever that is (lists of packed views measured 20 % slower)
  *   "max_large_chunk"    upper bound of the elements one shared descriptor of a large tensor covers: a
  *                   power of two in [4096, 2^24] (default 2^24; smaller values measured no faster)
  * Affects plans whose tensors are set after the call. */
@@ -182,6 +186,15 @@ int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float be
  * NULL): 1 = every stream aligned to its 64/128-bit vector. */
 int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
                   uint8_t* tensor_class, uint8_t* vector_ok);
+
+/* Host-only: how many leading elements of this tensor the layout gives to a short descriptor of their own so
+ * that the tiles behind them start where the streams meet 128-byte lines (and 1 KiB boundaries where they
+ * can): 0 for tensors under 8192 elements, for streams that are aligned already, when no count improves the
+ * alignment, and with option "align_heads" = 0; at most 511 otherwise.  The head's descriptors are counted
+ * among the small ones of fsadam_layout, and the tensor's class and vector_ok refer to what follows the head.
+ * The values a step writes do not depend on it.  No counterpart in the reference, whose chunks always start
+ * at element 0 (multi_tensor_apply.cuh:74-86). */
+int fsadam_head_elems(const FsAdamTensor* tensor, int precision_mode, int64_t* head);
 
 /* ---- gradient pass: what runs on the gradients BEFORE the step, in one read.
  * Replaces, for one rank's gradients on one device:

@@ -475,6 +475,51 @@ def _set_grads(params, step, seed=5):
         p.grad = (torch.randn(p.numel(), generator=gen) * 1e-3).to(device=p.device, dtype=p.dtype)
 
 
+@pytest.mark.parametrize("precision_name", ["FULL_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION", "PURE_FP16", "MIXED_PRECISION"])
+def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_device, precision_name):
+    """Parameters (and gradients) that are views packed back to back into one buffer start between cache
+    lines.  Their state is allocated the same number of elements past a 1 KiB boundary (modulo 512), so one
+    head aligns every stream; the values must be those of the same parameters allocated one by one, and
+    saving and loading the state must keep them."""
+    Adam, _, Precision = api
+    sizes = (9001, 33, 8192, 140003, 20000)
+    separate = _random_problem(precision_name, cuda_device, sizes)
+    dtype = separate[0].dtype
+    flat = torch.empty(sum(sizes) + 3, device=cuda_device, dtype=dtype)
+    flat_grad = torch.empty_like(flat)
+    packed, at = [], 3
+    for p in separate:
+        view = flat[at:at + p.numel()]
+        view.copy_(p.detach())
+        packed.append(view.requires_grad_())
+        at += p.numel()
+    opts = [Adam(ps, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name]) for ps in (separate, packed)]
+    for step in range(1, 4):
+        _set_grads(separate, step)
+        at = 3
+        for p, q in zip(separate, packed):
+            q.grad = flat_grad[at:at + p.numel()].copy_(p.grad)
+            at += p.numel()
+        for opt in opts:
+            opt.step(scale=2.0)
+    for p, q in zip(separate, packed):
+        assert torch.equal(p.detach(), q.detach())
+        for key in ("exp_avg", "exp_avg_sq"):
+            a, b = opts[0].state[p][key], opts[1].state[q][key]
+            assert torch.equal(a, b)
+            if precision_name != "MIXED_PRECISION" and q.numel() >= 8192 and q.data_ptr() % 128:
+                assert (b.data_ptr() // b.element_size() - q.data_ptr() // q.element_size()) % 512 == 0, "state not placed like its parameter"
+                assert b.is_contiguous() and b.shape == q.shape
+    blob = io.BytesIO()
+    torch.save(opts[1].state_dict(), blob)
+    blob.seek(0)
+    fresh = Adam(packed, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name])
+    fresh.load_state_dict(torch.load(blob, weights_only=True))
+    for q in packed:
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(fresh.state[q][key], opts[1].state[q][key])
+
+
 def test_list_walk_helper_is_loaded():
     from fairscale_amd import _rows
 

@@ -132,6 +132,110 @@ def test_layout_classes_and_descriptor_counts():
             _cabi.set_option(k, v)
 
 
+def head_of(t, mode):
+    out = ctypes.c_int64(-1)
+    _cabi.check(_cabi.lib().fsadam_head_elems(rows(t), mode, ctypes.byref(out)))
+    return out.value
+
+
+def test_heads_bring_the_tiles_onto_line_boundaries():
+    """The first elements of a tensor whose streams start off a cache line go to a descriptor of their own
+    (fake addresses, host-side planning only)."""
+    A = 0x7000_0000_0000
+    same = lambda off, n, mode: tuple(A + (k << 34) + off * (2 if half else 4) for k, half in enumerate(_halves(mode))) + (0, n)  # noqa: E731
+    F, MX, ME, P16 = _cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16
+    # aligned streams, short tensors: nothing to do
+    assert head_of(same(0, 1 << 20, F), F) == 0
+    assert head_of(same(256, 1 << 20, F), F) == 0  # fp32 streams 1 KiB in: aligned as well
+    assert head_of(same(3, 8191, F), F) == 0
+    # fp32 streams all 3 elements (12 bytes) past a 1 KiB boundary: 253 elements reach the next one
+    assert head_of(same(3, 8192, F), F) == 253
+    assert head_of(same(255, 8192, F), F) == 1
+    # fp16 p and g at 2 bytes an element, fp32 state at 4: a head that is a multiple of 512 elements away suits both
+    assert head_of(same(5, 100000, ME), ME) == 507
+    assert head_of(same(300, 100000, ME), ME) == 212
+    assert head_of(same(7, 100000, P16), P16) == 505
+    # MIXED_PRECISION: fp32 p, m, v, fp16 g and fp16 copy
+    t = same(9, 100000, MX)
+    t = t[:4] + (A + (5 << 34) + 9 * 2, t[5])
+    assert head_of(t, MX) == 503
+    # state allocated on its own (aligned), parameters and gradients 4 elements into a flat buffer: moving
+    # the tiles would take m and v off their lines, which costs more than it gains
+    assert head_of((A + 16, A + (1 << 34), A + (2 << 34), A + (3 << 34) + 16, 0, 100000), F) == 0
+    # the same with fp16 parameters and gradients (8 bytes in): the fp32 state carries more bytes per element
+    assert head_of((A + 8, A + (1 << 34), A + (2 << 34), A + (3 << 34) + 8, 0, 100000), ME) == 0
+    # only the gradient off its line: it follows the others
+    assert head_of((A, A + (1 << 34), A + (2 << 34), A + (3 << 34) + 16, 0, 100000), F) == 0
+    # the other way round, p, m, v 64 bytes in and the gradient aligned: the three heavier streams win
+    assert head_of((A + 64, A + (1 << 34) + 64, A + (2 << 34) + 64, A + (3 << 34), 0, 100000), F) == 240
+    old = _cabi.get_option("align_heads")
+    try:
+        _cabi.set_option("align_heads", 0)
+        assert head_of(same(3, 8192, F), F) == 0
+    finally:
+        _cabi.set_option("align_heads", old)
+
+
+def _halves(mode):
+    """which of p, m, v, g are fp16 in a mode"""
+    return {_cabi.FULL_PRECISION: (0, 0, 0, 0), _cabi.MIXED_PRECISION: (0, 0, 0, 1), _cabi.MEMORY_EFFICIENT_MIXED_PRECISION: (1, 0, 0, 1),
+            _cabi.PURE_FP16: (1, 1, 1, 1)}[mode]
+
+
+def test_no_other_head_would_align_better():
+    """The head is chosen among a handful of candidates (the counts that bring one stream onto a line or a
+    1 KiB boundary).  An exhaustive search over every count below 1024 with the same weights (bytes a
+    stream moves per element x 0 / 1 / 5 / 6 for 1 KiB-, line-, 16-byte- or element-aligned) must not find
+    a cheaper one, nor an equally cheap shorter one."""
+    rng = np.random.default_rng(77)
+    A = 0x7000_0000_0000
+    for case in range(300):
+        mode = [_cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16][case % 4]
+        sizes = [2 if h else 4 for h in _halves(mode)]
+        streams = [(A + (k << 34) + int(rng.integers(0, 512)) * sz * int(rng.choice([1, 1, 4, 32])), sz, (1 if k == 3 else 2) * sz)
+                   for k, sz in enumerate(sizes)]
+        copy = A + (5 << 34) + int(rng.integers(0, 512)) * 2 if mode == _cabi.MIXED_PRECISION else 0
+        if copy:
+            streams.append((copy, 2, 2))
+
+        def cost(head):
+            total = 0
+            for addr, sz, moved in streams:
+                a = addr + head * sz
+                total += moved * (0 if a % 1024 == 0 else 1 if a % 128 == 0 else 5 if a % 16 == 0 else 6)
+            return total
+
+        got = head_of((streams[0][0], streams[1][0], streams[2][0], streams[3][0], copy, 50000), mode)
+        best = min(range(1024), key=lambda h: (cost(h), h))
+        assert (cost(got), got) == (cost(best), best), (case, mode, [hex(s[0]) for s in streams], got, best)
+
+
+def test_layout_counts_heads_among_the_small_descriptors():
+    A = 0x7000_0000_0000
+    t = lambda n, off: (A + off, A + (1 << 34) + off, A + (2 << 34) + off, A + (3 << 34) + off, 0, n)  # noqa: E731
+    # 100 elements short of a 1 KiB boundary: head 100, then exactly two shared chunks
+    lay, cls, vec = layout([t(131072 + 100, 1024 - 400)], _cabi.FULL_PRECISION)
+    assert cls == [2] and vec == [1]
+    assert lay["n_large_descriptors"] == 2 and lay["n_small_descriptors"] == 1
+    # without the head the same tensor needs a third chunk
+    old = _cabi.get_option("align_heads")
+    try:
+        _cabi.set_option("align_heads", 0)
+        lay0, cls0, vec0 = layout([t(131072 + 100, 1024 - 400)], _cabi.FULL_PRECISION)
+        assert cls0 == [2] and vec0 == [1] and lay0["n_large_descriptors"] == 3 and lay0["n_small_descriptors"] == 0
+    finally:
+        _cabi.set_option("align_heads", old)
+    # a head can take a tensor below the size that shares descriptors, and can be longer than a tile
+    lay, cls, vec = layout([t(131072 + 10, 4)], _cabi.FULL_PRECISION)  # head 255, 130827 left
+    assert cls == [1] and vec == [1] and lay["n_large_descriptors"] == 0 and lay["n_small_descriptors"] == 1 + -(-130827 // 256)
+    half = lambda n, off: (A + off, A + (1 << 34) + off, A + (2 << 34) + off, A + (3 << 34) + off, 0, n)  # noqa: E731
+    lay, cls, vec = layout([half(9000, 2)], _cabi.PURE_FP16)  # 2 bytes in: head 511 halves, under one 512-element tile
+    assert lay["n_small_descriptors"] == 1 + -(-(9000 - 511) // 512) and vec == [1]
+    # vector_ok describes what follows the head: 3 elements in, the tiles start aligned
+    lay, cls, vec = layout([t(10000, 12), t(5000, 12)], _cabi.FULL_PRECISION)
+    assert vec == [1, 0]
+
+
 def test_layout_matches_a_python_model_on_drawn_lists():
     """Descriptor and workgroup counts for drawn lists, modes and options against ten lines of Python."""
     import random

@@ -160,6 +160,30 @@ def test_misaligned_views_and_device_resident_scale(cuda_device, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("write_back", [True, False])
+@pytest.mark.parametrize("align_heads", [1, 0])
+def test_heads_split_off_gradient_views_between_cache_lines(cuda_device, dtype, write_back, align_heads):
+    """Gradients of 8192 elements and more that start off a 1 KiB boundary give up their first elements to a
+    descriptor of their own (the tiles behind start aligned); what is stored, the flag and the maximum stay
+    exact and the sum of squares within its bar, with the option on and off, for views that start 1, 37 and
+    300 elements into their allocations, one of them with a non-finite value inside the head."""
+    from fairscale_amd import _cabi
+
+    for shift in (1, 37, 300):
+        host = host_grads(dtype, 12 + shift, [8191, 8192, 8193, 131072 + 200, 300001], scale=64.0)
+        _cabi.set_option("align_heads", align_heads)
+        try:
+            dev, stats, want = run_both(host, cuda_device, 1 / 64, write_back, misalign=shift)
+            check(host, dev, stats, want, f"shift {shift}")
+            bad = host_grads(dtype, 99, [20000], scale=64.0)
+            bad[0][3] = np.inf
+            dev, stats, want = run_both(bad, cuda_device, 1 / 64, write_back, misalign=shift)
+            assert want[0] == 1.0 and stats.found_inf.item() == 1.0
+        finally:
+            _cabi.set_option("align_heads", 1)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_non_finite_at_every_position_of_a_tile(cuda_device, dtype):
     """One inf or NaN at a time at every lane position of a 16-byte vector, at tile edges and in the
     ragged tail: flag up, norms inf/NaN, everything else still unscaled."""

@@ -151,6 +151,29 @@ def test_misaligned_views(oracle, cuda_device, mode, which, unaligned_vectors):
         _cabi.set_option("unaligned_vectors", 1)
 
 
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+@pytest.mark.parametrize("which", ["all", "p_and_g"])
+@pytest.mark.parametrize("align_heads", [1, 0])
+def test_heads_split_off_views_that_start_between_cache_lines(oracle, cuda_device, mode, which, align_heads):
+    """Tensors of 8192 elements and more whose streams start off a 128-byte line give up a head of up to 511
+    elements so that their tiles start on line boundaries; smaller ones and aligned ones do not.  Every
+    stream shifted by the same element count (views into flat buffers: a common head aligns them all),
+    or only p and g shifted (state allocated by the optimizer, parameters and gradients views): the
+    head's elements, the tiles behind it and the ragged end must all come out as the oracle's, with the
+    option on and off."""
+    from fairscale_amd import _cabi
+
+    sizes = [8191, 8192, 8193, 20000, 131071 + 300, 131072 + 511, 131072 + 512, 300001]
+    shifts = [4, 4, 36, 260, 100, 511, 5, 7]
+    names = ("p", "g", "m", "v", "p16") if which == "all" else ("p", "g", "p16")
+    _cabi.set_option("align_heads", align_heads)
+    try:
+        run_case(oracle, cuda_device, mode, sizes, 2, 4300 + mode, dict(DEFAULT, decay=0.01), grad_scale=1.0 if mode == FULL else 128.0,
+                 misalign={name: shifts for name in names}, optim_scale=65536.0 if mode == PURE16 else 1.0)
+    finally:
+        _cabi.set_option("align_heads", 1)
+
+
 def test_steps_alternating_between_streams(oracle, cuda_device):
     """Every step runs on another stream than the one before.  In the first half the gradient tensors stay
     where they are, so kernels on one stream read a table that was uploaded on another (the library
