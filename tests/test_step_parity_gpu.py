@@ -206,7 +206,8 @@ def test_steps_alternating_between_streams(oracle, cuda_device):
 def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
     """Differential test on drawn configurations: mode, list length, sizes around every boundary (empty,
     below a tile, tile multiples +-1, around the large-tensor threshold), a separate element offset for
-    every stream of every tensor, eps placement, bias correction, decay, power-of-two or odd scales;
+    every stream of every tensor (every third seed: up to 511 elements, shared by the streams or not),
+    eps placement, bias correction, decay, power-of-two or odd scales;
     every second seed also plants infinities, NaNs, the largest and the smallest magnitudes and zeros
     in the gradients of the second step."""
     import random
@@ -234,6 +235,11 @@ def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
         sizes.append(77)
     names = ["p", "m", "v", "g", "p16"]
     misalign = {name: [rng.choice([0, 0, 1, 2, 3, 5, 7]) for _ in sizes] for name in names}
+    if seed % 3 == 0:  # farther into the allocation: other heads in front of the aligned tiles (drawn apart, the sequence above stays)
+        far = random.Random(77000 + seed)
+        same = far.randrange(2) == 0  # one offset per tensor for every stream, or one per stream
+        per_tensor = [far.choice([0, 1, 33, 64, 130, 300, 511]) for _ in sizes]
+        misalign = {name: (per_tensor if same else [far.choice([0, 1, 33, 64, 130, 300, 511]) for _ in sizes]) for name in names}
     hyper = dict(lr=rng.choice([1e-3, 3e-2]), beta1=rng.choice([0.9, 0.5]), beta2=rng.choice([0.999, 0.95]),
                  eps=rng.choice([1e-8, 1e-3]), eps_mode=rng.randrange(2), bias_correction=rng.randrange(2),
                  decay=rng.choice([0.0, 0.01]))
