@@ -114,6 +114,11 @@ def lib() -> ctypes.CDLL:
         got = L.fsadam_version()
         if got != ABI_VERSION:
             raise ImportError(f"libfsadam.so has ABI version {got}, this package expects {ABI_VERSION}")
+        # The streams this package hands to the library are torch's, which live as long as the process, so
+        # the library may record its events only when something has to wait for them (3 us less per step).
+        # A caller that steps on a torch.cuda.ExternalStream it destroys later sets the option back to 0.
+        if L.fsadam_set_option(b"lazy_events", 1) != 0:
+            raise ImportError("libfsadam.so does not know the option lazy_events")
         _lib = L
     return _lib
 

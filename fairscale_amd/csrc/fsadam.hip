@@ -82,6 +82,7 @@ struct Options {
     int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
     int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
     int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
+    int64_t lazy_events = 0;        // 1: events behind steps are recorded only when needed (streams must outlive the plan)
     int64_t align_heads = 1;        // 1: a tensor whose streams start off a cache line gives up a short head so that the rest starts on one
 };
 
@@ -245,6 +246,20 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
 
 }  // namespace
 
+// "Everything enqueued so far that uses X" as something a stream or the host can wait for.  By default
+// the event is recorded right behind every use.  With option "lazy_events" it is only recorded when
+// somebody needs it (another stream takes over, the table slot is about to be overwritten, the plan
+// goes away), so that a step on the stream of the step before enqueues its kernel and nothing else
+// (3 us less per step); recording late marks a later point of the same stream, which covers the uses
+// as well, but it touches the stream after the call that used it has returned: the caller must then
+// keep every stream it has passed alive for as long as the plan (or the cache) lives.
+struct UseMark {
+    hipEvent_t event = nullptr;
+    hipStream_t stream = nullptr;  // where the uses were enqueued
+    bool used = false;             // there has been a use
+    bool pending = false;          // uses enqueued on `stream` since the event was last recorded
+};
+
 // A device table plus its pinned staging copy.  A plan keeps a small ring of them: when a pointer
 // of the list moves, the new table goes into the next slot, so the host only ever waits for the
 // step that used that slot kTableSlots updates ago, not for the step still in flight.
@@ -252,9 +267,7 @@ struct TableSlot {
     int64_t cap_descs = 0;
     ChunkDesc* d_table = nullptr;
     ChunkDesc* h_table = nullptr;  // pinned
-    hipEvent_t last_use = nullptr;
-    hipStream_t last_stream = nullptr;  // the stream last_use was recorded on
-    bool used = false;
+    UseMark mark;
 };
 constexpr int kTableSlots = 3;
 
@@ -272,26 +285,59 @@ struct FsAdamPlan {
 
 namespace {
 
+int mark_init(UseMark& m) {
+    if (!m.event) FS_HIP(hipEventCreateWithFlags(&m.event, hipEventDisableTiming));
+    return FSADAM_OK;
+}
+// A use has been enqueued on `stream` (after mark_order_after for that stream).
+int mark_use(UseMark& m, hipStream_t stream, bool lazy) {
+    m.stream = stream;
+    m.used = true;
+    m.pending = lazy;
+    if (!lazy) FS_HIP(hipEventRecord(m.event, stream));
+    return FSADAM_OK;
+}
+// Make the event cover every use enqueued so far.  A stream that cannot take the record any more (the
+// caller destroyed it) has nothing left in flight that a device-wide wait would not cover.
+int mark_settle(UseMark& m) {
+    if (!m.pending) return FSADAM_OK;
+    if (hipEventRecord(m.event, m.stream) != hipSuccess) {
+        (void)hipGetLastError();
+        FS_HIP(hipDeviceSynchronize());
+        m.used = false;
+    }
+    m.pending = false;
+    return FSADAM_OK;
+}
+// The host waits until every use has finished.
+int mark_wait(UseMark& m) {
+    const int rc = mark_settle(m);
+    if (rc) return rc;
+    if (m.used && m.event) FS_HIP(hipEventSynchronize(m.event));
+    return FSADAM_OK;
+}
+// Work about to be enqueued on `stream` is ordered after the uses so far when the caller has moved to
+// another stream; on one stream the order is already there.
+int mark_order_after(UseMark& m, hipStream_t stream) {
+    if (!m.used || m.stream == stream) return FSADAM_OK;
+    const int rc = mark_settle(m);
+    if (rc) return rc;
+    if (m.used) FS_HIP(hipStreamWaitEvent(stream, m.event, 0));
+    return FSADAM_OK;
+}
+void mark_destroy(UseMark& m) {
+    (void)mark_wait(m);
+    if (m.event) (void)hipEventDestroy(m.event);
+    m = UseMark();
+}
+
 void slot_release(TableSlot& slot) {
-    if (slot.used && slot.last_use) (void)hipEventSynchronize(slot.last_use);
+    (void)mark_wait(slot.mark);
     if (slot.d_table) (void)hipFree(slot.d_table);
     if (slot.h_table) (void)hipHostFree(slot.h_table);
     slot.d_table = slot.h_table = nullptr;
     slot.cap_descs = 0;
-    slot.used = false;
-}
-
-// Work that reads a table slot (or a plan's partial sums) is ordered after the upload or launch that
-// touched it last when the caller moves to another stream; on one stream the order is already there.
-int order_after(hipEvent_t last_use, bool used, hipStream_t last_stream, hipStream_t stream) {
-    if (used && last_use && last_stream != stream) FS_HIP(hipStreamWaitEvent(stream, last_use, 0));
-    return FSADAM_OK;
-}
-int slot_mark(TableSlot& slot, hipStream_t stream) {
-    FS_HIP(hipEventRecord(slot.last_use, stream));
-    slot.last_stream = stream;
-    slot.used = true;
-    return FSADAM_OK;
+    slot.mark.used = slot.mark.pending = false;
 }
 
 // The scalars of a step (step size, scales) travel by value in the kernel arguments and the table slots
@@ -395,8 +441,10 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
 
     // next slot of the ring; it may still be read by the step that used it last
     TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
-    if (!slot.last_use) FS_HIP(hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming));
-    if (slot.used) FS_HIP(hipEventSynchronize(slot.last_use));
+    rc = mark_init(slot.mark);
+    if (rc) return rc;
+    rc = mark_wait(slot.mark);
+    if (rc) return rc;
     if (n_descs > slot.cap_descs) {
         slot_release(slot);
         const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
@@ -429,8 +477,13 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     plan->rows.assign(tensors, tensors + n);
     if (n_descs > 0)
         FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
-    rc = slot_mark(slot, stream);
+    rc = mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
     if (rc) return rc;
+    // the steps that used the table this one replaces are all enqueued: their slot's event can be taken now
+    if (plan->current >= 0) {
+        rc = mark_settle(plan->slots[plan->current].mark);
+        if (rc) return rc;
+    }
     plan->current = (plan->current + 1) % kTableSlots;
     plan->uploads += 1;
     return FSADAM_OK;
@@ -465,11 +518,11 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     const Layout& L = plan->layout;
     const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
     TableSlot& slot = plan->slots[plan->current];
-    int rc = order_after(slot.last_use, slot.used, slot.last_stream, stream);
+    int rc = mark_order_after(slot.mark, stream);
     if (rc) return rc;
     rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, L.n_small_descs, log2k, plan->opt, s, found_inf, stream);
     if (rc) return rc;
-    return slot_mark(slot, stream);
+    return mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
 }
 
 
@@ -483,6 +536,7 @@ struct GradPlan {
     int64_t max_large_chunk = kMaxLargeChunk;
     int64_t unaligned_vectors = 1;
     int64_t align_heads = 1;
+    bool lazy_events = false;
     int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
     std::vector<FsGradTensor> rows;
     Layout layout;
@@ -490,9 +544,7 @@ struct GradPlan {
     int current = -1;
     GradPartial* d_partials = nullptr;  // [cap_partials] first stage, then [kReduceBlocks] second stage, then [1] total
     int64_t cap_partials = 0;
-    hipEvent_t last_use = nullptr;
-    hipStream_t last_stream = nullptr;
-    bool used = false;
+    UseMark partials_mark;  // the partial sums are shared by every call of the plan
     uint64_t lru = 0;
 };
 
@@ -540,22 +592,22 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
 }
 
 void grad_plan_free(GradPlan* plan) {
-    if (plan->used && plan->last_use) (void)hipEventSynchronize(plan->last_use);
+    mark_destroy(plan->partials_mark);
     for (TableSlot& slot : plan->slots) {
         slot_release(slot);
-        if (slot.last_use) (void)hipEventDestroy(slot.last_use);
+        mark_destroy(slot.mark);
     }
     if (plan->d_partials) (void)hipFree(plan->d_partials);
-    if (plan->last_use) (void)hipEventDestroy(plan->last_use);
     delete plan;
 }
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
 void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves,
-                int64_t* align_heads) {
+                int64_t* align_heads, int64_t* lazy_events) {
     std::lock_guard<std::mutex> lock(g_mutex);
     *align_heads = g_opt.align_heads;
+    *lazy_events = g_opt.lazy_events;
     // a pass that only reads pays for every small store it makes: 16 tiles share one partial
     *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
     *max_large_chunk = g_opt.max_large_chunk;
@@ -571,9 +623,12 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
     const int64_t n_descs = L.n_large_descs + L.n_small_descs;
     TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
-    if (!slot.last_use) FS_HIP(hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming));
-    if (!plan->last_use) FS_HIP(hipEventCreateWithFlags(&plan->last_use, hipEventDisableTiming));
-    if (slot.used) FS_HIP(hipEventSynchronize(slot.last_use));
+    int rc = mark_init(slot.mark);
+    if (rc) return rc;
+    rc = mark_init(plan->partials_mark);
+    if (rc) return rc;
+    rc = mark_wait(slot.mark);
+    if (rc) return rc;
     if (n_descs > slot.cap_descs) {
         slot_release(slot);
         const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
@@ -590,7 +645,8 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     }
     if (n_blocks + kReduceBlocks + 1 > plan->cap_partials) {
         // the partials may still be read by the reduction of the previous call
-        if (plan->used) FS_HIP(hipEventSynchronize(plan->last_use));
+        rc = mark_wait(plan->partials_mark);
+        if (rc) return rc;
         if (plan->d_partials) (void)hipFree(plan->d_partials);
         plan->d_partials = nullptr;
         plan->cap_partials = 0;
@@ -631,8 +687,12 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     plan->rows.assign(grads, grads + n);
     if (n_descs > 0)
         FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
-    const int rc = slot_mark(slot, stream);
+    rc = mark_use(slot.mark, stream, plan->lazy_events);
     if (rc) return rc;
+    if (plan->current >= 0) {
+        rc = mark_settle(plan->slots[plan->current].mark);
+        if (rc) return rc;
+    }
     plan->current = (plan->current + 1) % kTableSlots;
     return FSADAM_OK;
 }
@@ -648,9 +708,9 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     GradPartial* first = plan->d_partials;
     GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
     GradPartial* total = second + kReduceBlocks;
-    int rc = order_after(slot.last_use, slot.used, slot.last_stream, stream);
+    int rc = mark_order_after(slot.mark, stream);
     if (rc) return rc;
-    rc = order_after(plan->last_use, plan->used, plan->last_stream, stream);  // the partial sums are shared by every call
+    rc = mark_order_after(plan->partials_mark, stream);
     if (rc) return rc;
     // workgroups of `waves` consecutive tiles, one partial each
     const int64_t waves = plan->waves;
@@ -682,12 +742,9 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total, 1, (int)(sizeof(T) == 2),
                        found_inf, sum_squares, abs_max);
     FS_HIP(hipGetLastError());
-    rc = slot_mark(slot, stream);
+    rc = mark_use(slot.mark, stream, plan->lazy_events);
     if (rc) return rc;
-    FS_HIP(hipEventRecord(plan->last_use, stream));
-    plan->last_stream = stream;
-    plan->used = true;
-    return FSADAM_OK;
+    return mark_use(plan->partials_mark, stream, plan->lazy_events);
 }
 
 std::vector<GradPlan*> g_grad_cache;
@@ -761,6 +818,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "align_heads") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "align_heads must be 0 or 1");
         g_opt.align_heads = value;
+    } else if (k == "lazy_events") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "lazy_events must be 0 or 1");
+        g_opt.lazy_events = value;
     } else if (k == "max_large_chunk") {
         if (value < 4096 || value > kMaxLargeChunk || (value & (value - 1)) != 0)
             return fail(FSADAM_EINVAL, "max_large_chunk must be a power of two in [4096, 2^24] elements");
@@ -791,6 +851,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "max_large_chunk") *value = g_opt.max_large_chunk;
     else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
     else if (k == "align_heads") *value = g_opt.align_heads;
+    else if (k == "lazy_events") *value = g_opt.lazy_events;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else if (k == "grad_waves") *value = g_opt.grad_waves;
@@ -896,8 +957,7 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
 int fsadam_plan_destroy(FsAdamPlan* plan) {
     if (!plan) return FSADAM_OK;
     plan_release_buffers(plan);
-    for (TableSlot& slot : plan->slots)
-        if (slot.last_use) (void)hipEventDestroy(slot.last_use);
+    for (TableSlot& slot : plan->slots) mark_destroy(slot.mark);
     delete plan;
     return FSADAM_OK;
 }
@@ -963,9 +1023,9 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads;
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy;
     grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
-               &cur_waves, &cur_heads);
+               &cur_waves, &cur_heads, &cur_lazy);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
@@ -997,12 +1057,14 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->max_large_chunk = cur_chunk;
         victim->unaligned_vectors = cur_unaligned;
         victim->align_heads = cur_heads;
+        victim->lazy_events = cur_lazy != 0;
         victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;
     }
     hit->lru = ++g_tick;
+    hit->lazy_events = cur_lazy != 0;
     return grad_dtype == FSADAM_GRAD_F16
                ? grad_plan_run<_Float16>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream)
                : grad_plan_run<float>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream);

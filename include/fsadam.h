@@ -127,6 +127,12 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   into a flat buffer) gives its first elements, at most 511, to a short descriptor of their own, so
  *                   that every tile behind them starts on line boundaries (see fsadam_head_elems); 0: tiles start
  *                   at element 0 wherever that is (lists of packed views measured 20 % slower)
+ *   "lazy_events"   0 (default): an event is recorded behind every step (and gradient pass); it is what the library
+ *                   waits for before it overwrites a table a step may still read, and what orders a call on
+ *                   another stream behind the one before.  1: the event is only recorded when one of those needs
+ *                   it, which makes a step 3 us shorter, but touches the stream after the call that used it has
+ *                   returned: every stream ever passed must then stay alive until the plan is destroyed (for
+ *                   fsadam_step / fsadam_grad_pass: until fsadam_clear_cache)
  *   "max_large_chunk"    upper bound of the elements one shared descriptor of a large tensor covers: a
  *                   power of two in [4096, 2^24] (default 2^24; smaller values measured no faster)
  * Affects plans whose tensors are set after the call. */

@@ -276,7 +276,7 @@ def options():
     """Set tuning options for one test and put the defaults back afterwards."""
     from fairscale_amd import _cabi
 
-    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors")
+    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events")
     old = {k: _cabi.get_option(k) for k in names}
 
     def set_many(**kw):
@@ -307,6 +307,36 @@ def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, opti
     for mode in (MEMEFF, PURE16):
         run_case(oracle, cuda_device, mode, [5, 4099, 40000, 140001, 524288 + 17], 2, 4900 + mode, DEFAULT, grad_scale=8.0,
                  optim_scale=65536.0 if mode == PURE16 else 1.0)
+
+
+@pytest.mark.parametrize("lazy_events", [0, 1])
+def test_event_bookkeeping_eager_and_lazy(oracle, cuda_device, options, lazy_events):
+    """The event behind a step is what protects a table that may still be read and what orders a step on
+    another stream behind the one before.  Recorded behind every step (the library's default) or only when
+    needed (what this package switches on, torch's streams being immortal), the results are the same:
+    steps hopping between three streams without any synchronisation by the caller, with the gradient
+    pointers moving every step (a new table every step, the ring of slots wrapping around)."""
+    from fairscale_amd import fused_adam_hip
+
+    options(lazy_events=lazy_events)
+    host = C.Tensors(FULL, [5, 4099, 140001, 70000], 5100)
+    dev = GpuList(host, cuda_device)
+    streams = [torch.cuda.Stream(cuda_device) for _ in range(3)]
+    flag = np.zeros(1, np.float32)
+    plan = fused_adam_hip.TensorListPlan(FULL, cuda_device)
+    keep = []
+    for step in range(1, 13):
+        grads = host.grads(step)
+        g = to_gpu(grads, cuda_device)  # fresh allocations: the pointers move
+        keep.append(g)
+        torch.cuda.synchronize(cuda_device)  # the gradients were written on the default stream
+        with torch.cuda.stream(streams[(step * 2) % 3]):
+            plan.step([dev.p, dev.m, dev.v, g], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, dev.found_inf, step, 1, 1, 0.0)
+        oracle_step(oracle, host, grads, flag, **dict(DEFAULT, step=step))
+    torch.cuda.synchronize(cuda_device)
+    compare(host, dev, f"lazy_events={lazy_events}")
+    assert plan.info()["uploads"] == 12
+    plan.close()
 
 
 def test_pointer_changes_while_earlier_steps_are_in_flight(oracle, cuda_device):
