@@ -7,6 +7,7 @@ the kernels run on torch's current HIP stream and the call does not wait for the
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import List, Optional, Sequence
 
@@ -135,8 +136,23 @@ def _rows_ptr(rows: np.ndarray):
     return rows.ctypes.data_as(ctypes.POINTER(_cabi.FsAdamTensor))
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_SAME_DEVICE = contextlib.nullcontext()
+
+
 def _stream_handle(device: torch.device) -> int:
+    """hipStream_t of torch's current stream on ``device`` (without building a Stream object when torch
+    offers the raw handle: this runs once per step)."""
+    if _raw_stream is not None and device.index is not None:
+        return int(_raw_stream(device.index))
     return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _on_device(device: torch.device):
+    """Context that makes ``device`` current for the native call; nothing to do when it already is."""
+    if device.index is not None and torch.cuda.current_device() == device.index:
+        return _SAME_DEVICE
+    return torch.cuda.device(device)
 
 
 def adam(chunk_size: int, noop_flag: Optional[torch.Tensor], tensor_lists: List[List[torch.Tensor]], lr: float,
@@ -157,7 +173,7 @@ def adam(chunk_size: int, noop_flag: Optional[torch.Tensor], tensor_lists: List[
     if found_inf.device != device:
         raise RuntimeError("found_inf must live on the tensors' device")
     L = _cabi.lib()
-    with torch.cuda.device(device):
+    with _on_device(device):
         _cabi.check(L.fsadam_step(_rows_ptr(rows), rows.shape[0], precision, lr, beta1, beta2, eps, grad_scale,
                                   optim_scale, decay, int(step), int(mode), int(bias_correction),
                                   found_inf.data_ptr(), _stream_handle(device)))
@@ -219,7 +235,7 @@ class TensorListPlan:
         scale_on_device = isinstance(grad_scale, torch.Tensor)
         if scale_on_device and (grad_scale.dtype != torch.float32 or grad_scale.numel() != 1 or grad_scale.device != self.device):
             raise RuntimeError("a tensor scale must be float32 with one element on the parameters' device")
-        with torch.cuda.device(self.device):
+        with _on_device(self.device):
             stream = _stream_handle(self.device)
             if changed or self._dirty:
                 _cabi.check(L.fsadam_plan_set_tensors(self._handle, _rows_ptr(rows), rows.shape[0], stream))
