@@ -12,6 +12,7 @@ Deliberate differences, all supersets of the reference behaviour:
   ``tests/optim/test_adam.py:357-370`` expects.
 * The device flag is only allocated, cleared and read back in PURE_FP16: the other three modes cannot
   raise it (fused_adam_cuda_kernel.cu:94-105 is the only writer), so they step without a host sync.
+  In PURE_FP16 it is cleared only after a step that raised it (a flag read back as 0 is still 0).
   The scale bookkeeping they do every step (adam.py:289-295) is kept.
 * After an overflow m and v are zeroed in place rather than re-allocated (adam.py:285-288), and
   parameters that never had a gradient keep an empty state instead of a half-initialised one.
@@ -245,11 +246,29 @@ class Adam(torch.optim.Optimizer):
         self._group_cache = {}
 
     def _flag_for(self, device: torch.device) -> torch.Tensor:
+        """The overflow flag of a device, holding 0.  The kernel only ever raises it, so it is cleared
+        again only after a step that raised it (or whose result was never read): a step that read back 0
+        leaves it ready for the next one.  (The reference allocates a fresh zero flag per group and
+        step, adam.py:256.)"""
+        unread = self.__dict__.setdefault("_flags_unread", set())
         flag = self._flags.get(device)
         if flag is None:
             flag = torch.zeros(1, dtype=torch.float32, device=device)
             self._flags[device] = flag
+        elif device in unread:
+            flag.zero_()
+        unread.add(device)
         return flag
+
+    def _read_flags(self, flags: List[torch.Tensor]) -> bool:
+        """adam.py:278: did any device raise its flag?  One blocking read per flag, as in the reference."""
+        raised = False
+        for flag in flags:
+            if flag.item() != 0.0:
+                raised = True
+            else:
+                self._flags_unread.discard(flag.device)
+        return raised
 
     def attach_fp16_copies(self, copies: Optional[Dict[torch.Tensor, torch.Tensor]]) -> None:
         """FULL_PRECISION only.  ``copies`` maps parameters to fp16 tensors of the same shape that the
@@ -436,7 +455,6 @@ class Adam(torch.optim.Optimizer):
                 flag = None
                 if watch_overflow:
                     flag = self._flag_for(plan.device)
-                    flag.zero_()
                     flags.append(flag)
                 plan.step_rows(table_changed, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
                                step_no, self.eps_mode, bias_correction, group["weight_decay"])
@@ -452,13 +470,12 @@ class Adam(torch.optim.Optimizer):
                 flag = None
                 if watch_overflow:
                     flag = self._flag_for(device)
-                    flag.zero_()
                     flags.append(flag)
                 self._plan_for(gi, device, native_mode).step(
                     lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag, step_no, self.eps_mode,
                     bias_correction, group["weight_decay"])
 
-            overflowed = bool(sum(f.item() for f in flags)) if flags else False  # adam.py:278
+            overflowed = self._read_flags(flags) if flags else False  # adam.py:278
             if overflowed:
                 self._steps_since_optim_scale_change = 0
                 self._optim_scale /= 2
