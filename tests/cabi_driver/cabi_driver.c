@@ -41,8 +41,12 @@ int fsadam_oracle_step(int mode, void* p, void* m, void* v, const void* g, void*
         }                                                                                \
     } while (0)
 
-enum { N_TENSORS = 7, N_STEPS = 4 };
-static const int64_t kSizes[N_TENSORS] = {1, 255, 256, 257, 0, 70001, 300000};
+enum { N_TENSORS = 9, N_STEPS = 4 };
+static const int64_t kSizes[N_TENSORS] = {1, 255, 256, 257, 0, 70001, 300000, 20000, 140000};
+/* elements between the start of an allocation and the tensor: the last two are views that start between
+ * cache lines, as views packed into a flat buffer do (the layout gives their first elements a descriptor of
+ * their own) */
+static const int64_t kShift[N_TENSORS] = {0, 0, 0, 0, 0, 0, 0, 5, 301};
 
 static uint64_t g_state = 0x9e3779b97f4a7c15ull;
 static float uniform_pm1(void) { /* xorshift64*: deterministic, in (-1, 1) */
@@ -64,7 +68,7 @@ static void fill(void* dst, int64_t n, int is_half, float scale) {
 }
 
 typedef struct {
-    void *h[5], *d[5]; /* p, m, v, g, p_copy: host (oracle) and device copies */
+    void *h[5], *d[5], *base[5]; /* p, m, v, g, p_copy: host (oracle) copy, device tensor, device allocation */
 } Streams;
 
 static int run_mode(int mode, const char* name) {
@@ -90,7 +94,8 @@ static int run_mode(int mode, const char* name) {
             if (s == 4 && !has_copy) continue;
             const size_t bytes = (size_t)(n > 0 ? n : 1) * elem_size(half_of[s]);
             t[i].h[s] = calloc(1, bytes);
-            CHECK_HIP(hipMalloc(&t[i].d[s], bytes));
+            CHECK_HIP(hipMalloc(&t[i].base[s], bytes + (size_t)kShift[i] * elem_size(half_of[s])));
+            t[i].d[s] = (char*)t[i].base[s] + (size_t)kShift[i] * elem_size(half_of[s]);
             if (s == 0) fill(t[i].h[s], n, half_of[s], 0.02f);
             CHECK_HIP(hipMemcpy(t[i].d[s], t[i].h[s], bytes, hipMemcpyHostToDevice));
         }
@@ -100,6 +105,25 @@ static int run_mode(int mode, const char* name) {
         rows[i].g = t[i].d[3];
         rows[i].p_copy = t[i].d[4];
         rows[i].numel = n;
+    }
+    /* every stream of a shifted tensor is off its lines by the same number of elements, so one head brings all
+     * of them onto 1 KiB boundaries; a tensor that starts on them keeps its first element */
+    for (int i = 0; i < N_TENSORS; ++i) {
+        int64_t head = -1;
+        CHECK_FS(fsadam_head_elems(&rows[i], mode, &head));
+        if (kSizes[i] < 8192) {
+            if (head != 0) { fprintf(stderr, "%s: tensor %d: head %lld on a short tensor\n", name, i, (long long)head); return 5; }
+            continue;
+        }
+        for (int s = 0; s < 5; ++s) {
+            if (!t[i].d[s]) continue;
+            const uintptr_t start = (uintptr_t)t[i].d[s] + (uintptr_t)head * elem_size(half_of[s]);
+            if (head < 0 || head > 511 || start % 1024 != 0) {
+                fprintf(stderr, "%s: tensor %d stream %d: head %lld leaves it at %#llx\n", name, i, s, (long long)head, (unsigned long long)start);
+                return 5;
+            }
+        }
+        if ((kShift[i] == 0) != (head == 0)) { fprintf(stderr, "%s: tensor %d: shift %lld, head %lld\n", name, i, (long long)kShift[i], (long long)head); return 5; }
     }
     FsAdamPlan* plan = NULL;
     CHECK_FS(fsadam_plan_create(mode, &plan));
@@ -144,7 +168,7 @@ static int run_mode(int mode, const char* name) {
     CHECK_FS(fsadam_plan_destroy(plan));
     for (int i = 0; i < N_TENSORS; ++i)
         for (int s = 0; s < 5; ++s) {
-            if (t[i].d[s]) CHECK_HIP(hipFree(t[i].d[s]));
+            if (t[i].base[s]) CHECK_HIP(hipFree(t[i].base[s]));
             free(t[i].h[s]);
         }
     CHECK_HIP(hipFree(d_flag));
@@ -234,5 +258,6 @@ int main(void) {
     bad |= run_grad_pass();
     if (fsadam_clear_cache() != FSADAM_OK) bad |= 1;
     printf(bad ? "FAILED\n" : "all modes bit-identical to the oracle\n");
+    fflush(stdout); /* the verdict must not depend on how the runtime's own exit handlers fare */
     return bad;
 }
