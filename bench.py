@@ -106,12 +106,14 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
     return out
 
 
-def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=False):
+def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=False, moving=False):
     """4096 fp32 tensors of log-uniform sizes (numel = max(1, round(2**U(0, 20)))), FULL_PRECISION with weight
     decay and eps inside the square root: the list-handling case.  Host time per step (the calls return
     without waiting), device time per step, and wall time of back-to-back steps.  ``packed``: the
     parameters are views laid back to back into one flat buffer that starts one element in (so nearly every
-    tensor starts between cache lines), the gradients likewise."""
+    tensor starts between cache lines), the gradients likewise.  ``moving``: every step finds the gradients in
+    other tensors than the step before (two sets taking turns, as when ``zero_grad(set_to_none=True)`` lets the
+    allocator hand out other blocks), so the descriptor table is rebuilt and sent again every step."""
     import random
 
     from fairscale_amd import _rows
@@ -132,14 +134,22 @@ def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=F
         for p in params:
             p.grad = torch.empty_like(p).normal_(0, 1e-3)
     opt = Adam(params, lr=1e-3, weight_decay=0.01, eps_inside_sqrt=True, precision=Precision.FULL_PRECISION)
-    for _ in range(warmup):
+    sets = [[p.grad for p in params], [torch.empty_like(p).normal_(0, 1e-3) for p in params]] if moving else None
+
+    def one_step(i):
+        if moving:
+            for p, g in zip(params, sets[i % 2]):
+                p.grad = g
         opt.step()
+
+    for i in range(warmup):
+        one_step(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(steps):
-        opt.step()
+    for i in range(steps):
+        one_step(warmup + i)
     e1.record()
     host = time.perf_counter() - t0
     torch.cuda.synchronize()
@@ -151,7 +161,7 @@ def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=F
            "achieved_gbs": total * 28 * steps / wall / 1e9, "frac_of_hbm_peak": total * 28 * steps / wall / 1e9 / HBM_PEAK_GBS,
            "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "uploads": plan["uploads"],
            "list_walk": "c++" if _rows.native is not None else "python"}
-    del opt, params
+    del opt, params, sets
     torch.cuda.empty_cache()
     return out
 
@@ -264,6 +274,7 @@ def main():
         also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
         also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device)
         also["ragged_4096_packed_views_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device, packed=True)
+        also["ragged_4096_moving_gradients_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device, moving=True)
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"

@@ -17,7 +17,7 @@ MEMORY_EFFICIENT_MIXED_PRECISION = 2
 PURE_FP16 = 3
 FULL_PRECISION_FP16_COPY = 4
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
 
@@ -58,7 +58,8 @@ class FsAdamLayout(_Int64Fields):
     _fields_ = [
         (name, ctypes.c_int64)
         for name in ("tile_elems", "large_chunk_elems", "n_large_tensors", "n_small_tensors", "n_empty_tensors",
-                     "n_large_descriptors", "n_small_descriptors", "grid_large", "grid_small")
+                     "n_large_descriptors", "n_small_descriptors", "grid_large", "grid_small", "mid_chunk_elems", "n_mid_tensors",
+                     "n_mid_descriptors", "grid_mid")
     ]
 
 

@@ -176,13 +176,11 @@ __device__ __forceinline__ uint32_t tile_any(const ChunkDesc& d, uint32_t off, c
     return tile_elementwise<MODE, BLOCK, EPS_MODE, FAST_SCALES>(d, off, left < kTile ? left : kTile, s);
 }
 
-// One workgroup = one tile.  The first `n_large_blocks` tiles belong to the descriptors of large
-// tensors, 2^log2k tiles each; every tile after them has a descriptor of its own (small tensors),
-// stored behind the `n_large_descs` large ones.  `n_blocks`: tiles really launched for (the grid may
+// One workgroup = one tile, which finds its descriptor through `map` (large tensors, middle-sized
+// ones, then one descriptor per tile).  `n_blocks`: tiles really launched for (the grid may
 // be padded for the XCD remap).
 template <int MODE, int BLOCK, int GROUPS>
-__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
-                                                      uint32_t n_large_descs, uint32_t n_blocks, uint32_t xcd_stride,
+__global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restrict__ table, TileMap map, uint32_t n_blocks, uint32_t xcd_stride,
                                                       StepScalars s, float* __restrict__ found_inf) {
     constexpr uint32_t kTile = BLOCK * ModeTraits<MODE>::kElems * GROUPS;
 
@@ -195,9 +193,8 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
         block = group * 8u * xcd_stride + (in_group & 7u) * xcd_stride + (in_group >> 3);
         if (block >= n_blocks) return;
     }
-    const bool large = block < n_large_blocks;  // uniform: scalar selects
-    const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
-    const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
+    uint32_t chunk, off;
+    locate_tile(map, block, kTile, chunk, off);
     // The whole 64-byte descriptor in ONE scalar load (uniform address, constant address space), before
     // anything is tested: reading the count first and the pointers afterwards would put two memory
     // latencies in front of the first data load.
@@ -209,7 +206,7 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
     // scalar load at a uniform address, issued next to the descriptor's.  The host has already switched
     // to true division (fast_scales = 0), which gives the bits of a host-side scale of the same value.
     if (s.grad_scale_dev) s.grad_scale = *(const __attribute__((address_space(4))) float*)s.grad_scale_dev;
-    if (off >= d.n) return;  // tile past the end of its tensor (large tensors only)
+    if (off >= d.n) return;  // tile past the end of its tensor (shared descriptors only)
 
     uint32_t bad;
     if (s.eps_mode == 0) {

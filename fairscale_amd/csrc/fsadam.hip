@@ -22,10 +22,10 @@
 // The tensor list becomes a device-resident table of 64-byte chunk descriptors (five pointers
 // already advanced to the chunk, element count, alignment flag), uploaded once and reused every
 // step.  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
-// tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles; small tensors get
-// one descriptor per tile, placed after the large ones, so ONE launch covers any number of tensors
-// (the reference needs a launch per 36 tensors / 320 chunks because its table travels by value in
-// the kernel arguments).  Ragged tiles (the end of a tensor) take an element-wise path with the same
+// tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles, middle-sized ones
+// among 16, small ones get one descriptor per tile, each class placed after the one before, so ONE
+// launch covers any number of tensors (the reference needs a launch per 36 tensors / 320 chunks
+// because its table travels by value in the kernel arguments).  Ragged tiles (the end of a tensor) take an element-wise path with the same
 // arithmetic; full tiles of a tensor whose streams are only element-aligned use the same vector
 // instructions at odd addresses.
 //
@@ -82,6 +82,7 @@ struct Options {
     int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
     int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
     int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
+    int64_t mid_tiles = 16;         // tiles that share a descriptor of a middle-sized tensor (a power of two up to 64; 0 = no such class)
     int64_t lazy_events = 0;        // 1: events behind steps are recorded only when needed (streams must outlive the plan)
     int64_t align_heads = 1;        // 1: a tensor whose streams start off a cache line gives up a short head so that the rest starts on one
 };
@@ -206,17 +207,49 @@ int log2_exact(int64_t x) {
 struct Layout {
     int64_t tile_elems = 0;
     int64_t large_chunk_elems = 0;
-    int64_t n_large = 0, n_small = 0, n_empty = 0;
-    int64_t n_large_descs = 0, n_small_descs = 0;
+    int64_t mid_chunk_elems = 0;  // 0: no middle class
+    int64_t n_large = 0, n_mid = 0, n_small = 0, n_empty = 0;
+    int64_t n_large_descs = 0, n_mid_descs = 0, n_small_descs = 0;
     int64_t total_elems = 0;
     int64_t n_vector = 0, n_scalar = 0;
+
+    int64_t large_blocks() const { return n_large_descs * (large_chunk_elems / tile_elems); }
+    int64_t mid_blocks() const { return mid_chunk_elems ? n_mid_descs * (mid_chunk_elems / tile_elems) : 0; }
+    int64_t blocks() const { return tile_elems ? large_blocks() + mid_blocks() + n_small_descs : 0; }
+    int64_t descs() const { return n_large_descs + n_mid_descs + n_small_descs; }
 };
 
 int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// What is left of a tensor behind its head goes to shared descriptors of large_chunk_elems (class 2), of
+// mid_chunk_elems (class 3) or to one descriptor per tile (class 1).
+enum { kClassSmall = 1, kClassLarge = 2, kClassMid = 3 };
+int class_of(int64_t body, const Layout& L) {
+    if (body >= kLargeThreshold) return kClassLarge;
+    if (L.mid_chunk_elems > 0 && body >= L.mid_chunk_elems) return kClassMid;
+    return kClassSmall;
+}
+// A middle class only where its chunks stay well under the size that makes a tensor large.
+int64_t mid_chunk_for(int64_t tile_elems, int64_t mid_tiles) {
+    const int64_t chunk = tile_elems * mid_tiles;
+    return (mid_tiles > 1 && 2 * chunk <= kLargeThreshold) ? chunk : 0;
+}
+// The launch's view of a layout.
+TileMap tile_map(const Layout& L) {
+    TileMap map;
+    map.log2_large = (uint32_t)log2_exact(L.large_chunk_elems / L.tile_elems);
+    map.n_large_descs = (uint32_t)L.n_large_descs;
+    map.n_large_blocks = (uint32_t)L.large_blocks();
+    map.log2_mid = L.mid_chunk_elems ? (uint32_t)log2_exact(L.mid_chunk_elems / L.tile_elems) : 0u;
+    map.n_mid_descs = (uint32_t)L.n_mid_descs;
+    map.n_mid_blocks = (uint32_t)L.mid_blocks();
+    return map;
+}
+
 Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Options& opt) {
     Layout L;
     L.tile_elems = opt.block * mode_elems(mode) * opt.groups;
+    L.mid_chunk_elems = mid_chunk_for(L.tile_elems, opt.mid_tiles);
     int64_t min_large = 0;
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = tensors[t].numel;
@@ -224,11 +257,12 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
         if (numel == 0) { L.n_empty += 1; continue; }
         const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
         (row_vector_ok(tensors[t], mode, head) ? L.n_vector : L.n_scalar) += 1;
-        if (body >= kLargeThreshold) {
+        const int cls = class_of(body, L);
+        if (cls == kClassLarge) {
             L.n_large += 1;
             if (min_large == 0 || body < min_large) min_large = body;
         } else {
-            L.n_small += 1;
+            (cls == kClassMid ? L.n_mid : L.n_small) += 1;
         }
     }
     // every large tensor spans at least two chunks, so the empty tiles after its end stay a small share
@@ -238,7 +272,9 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
         if (numel == 0) continue;
         const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
         L.n_small_descs += ceil_div(head, L.tile_elems);
-        if (body >= kLargeThreshold) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        const int cls = class_of(body, L);
+        if (cls == kClassLarge) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        else if (cls == kClassMid) L.n_mid_descs += ceil_div(body, L.mid_chunk_elems);
         else L.n_small_descs += ceil_div(body, L.tile_elems);
     }
     return L;
@@ -375,10 +411,8 @@ int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t star
 }
 
 template <int MODE, int BLOCK, int GROUPS>
-int launch_tiles(const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
-                 const StepScalars& s, float* found_inf, hipStream_t stream) {
-    const int64_t n_large_blocks = n_large_descs << log2k;
-    const int64_t n_blocks = n_large_blocks + n_small_descs;
+int launch_tiles(const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf, hipStream_t stream) {
+    const int64_t n_blocks = L.blocks();
     if (n_blocks == 0) return FSADAM_OK;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
     uint32_t grid = (uint32_t)n_blocks, xcd_stride = 0;
@@ -386,34 +420,32 @@ int launch_tiles(const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_
         xcd_stride = (uint32_t)std::min<int64_t>(opt.xcd_remap, ceil_div(n_blocks, 8));
         grid = (uint32_t)(ceil_div(n_blocks, 8 * (int64_t)xcd_stride) * 8 * xcd_stride);
     }
-    hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table,
-                       (uint32_t)log2k, (uint32_t)n_large_blocks, (uint32_t)n_large_descs, (uint32_t)n_blocks, xcd_stride, s,
-                       found_inf);
+    hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table, tile_map(L),
+                       (uint32_t)n_blocks, xcd_stride, s, found_inf);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
 
 template <int MODE>
-int launch_shape(const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
-                 const StepScalars& s, float* found_inf, hipStream_t stream) {
+int launch_shape(const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf, hipStream_t stream) {
 #define FS_CASE(B, G)                      \
     if (opt.block == B && opt.groups == G) \
-    return launch_tiles<MODE, B, G>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream)
+    return launch_tiles<MODE, B, G>(table, L, opt, s, found_inf, stream)
     FS_CASE(64, 1); FS_CASE(64, 2); FS_CASE(128, 1); FS_CASE(128, 2); FS_CASE(256, 1); FS_CASE(256, 2);
 #undef FS_CASE
     return fail(FSADAM_EINVAL, "unsupported block/groups combination");
 }
 
-int launch_mode(int mode, const ChunkDesc* table, int64_t n_large_descs, int64_t n_small_descs, int log2k, const Options& opt,
-                const StepScalars& s, float* found_inf, hipStream_t stream) {
+int launch_mode(int mode, const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf,
+                hipStream_t stream) {
 #define FS_MODE(M) \
-    case M: return launch_shape<M>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream)
+    case M: return launch_shape<M>(table, L, opt, s, found_inf, stream)
     switch (mode) {
         FS_MODE(FSADAM_FULL_PRECISION);
         FS_MODE(FSADAM_MIXED_PRECISION);
         FS_MODE(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION);
         FS_MODE(FSADAM_FULL_PRECISION_FP16_COPY);
-        default: return launch_shape<FSADAM_PURE_FP16>(table, n_large_descs, n_small_descs, log2k, opt, s, found_inf, stream);
+        default: return launch_shape<FSADAM_PURE_FP16>(table, L, opt, s, found_inf, stream);
     }
 #undef FS_MODE
 }
@@ -435,9 +467,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     }
     if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
     const Layout L = compute_layout(tensors, n, plan->mode, plan->opt);
-    const int64_t n_descs = L.n_large_descs + L.n_small_descs;
-    if (L.n_large_descs * (L.large_chunk_elems / L.tile_elems) + L.n_small_descs > 0x7ffffff0)
-        return fail(FSADAM_EINVAL, "tensor list too large for one launch");
+    const int64_t n_descs = L.descs();
+    if (L.blocks() > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
     // next slot of the ring; it may still be read by the step that used it last
     TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
@@ -459,19 +490,22 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
         }
         slot.cap_descs = cap;
     }
-    // descriptors of large tensors first, then those of small ones: one launch covers both
+    // descriptors of large tensors first, then the middle-sized ones, then one per tile: one launch covers all
     ChunkDesc* large = slot.h_table;
-    ChunkDesc* small = slot.h_table + L.n_large_descs;
+    ChunkDesc* mid = large + L.n_large_descs;
+    ChunkDesc* small = mid + L.n_mid_descs;
     for (int64_t t = 0; t < n; ++t) {
         const FsAdamTensor& r = tensors[t];
         if (r.numel == 0) continue;
         const int64_t head = head_elems(r, plan->mode, plan->opt), body = r.numel - head;
         const bool vec = plan->opt.unaligned_vectors != 0 || row_vector_ok(r, plan->mode, head);
         small += fill_descs(small, r, plan->mode, 0, head, L.tile_elems, plan->opt.unaligned_vectors != 0);
-        if (body >= kLargeThreshold) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems, vec);
+        const int cls = class_of(body, L);
+        if (cls == kClassLarge) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems, vec);
+        else if (cls == kClassMid) mid += fill_descs(mid, r, plan->mode, head, body, L.mid_chunk_elems, vec);
         else small += fill_descs(small, r, plan->mode, head, body, L.tile_elems, vec);
     }
-    if (large != slot.h_table + L.n_large_descs || small != slot.h_table + n_descs)
+    if (large != slot.h_table + L.n_large_descs || mid != slot.h_table + L.n_large_descs + L.n_mid_descs || small != slot.h_table + n_descs)
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(tensors, tensors + n);
@@ -516,11 +550,10 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     s.fast_scales = (gs_ok && (plan->mode != FSADAM_PURE_FP16 || os_ok)) ? 1 : 0;
 
     const Layout& L = plan->layout;
-    const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
     TableSlot& slot = plan->slots[plan->current];
     int rc = mark_order_after(slot.mark, stream);
     if (rc) return rc;
-    rc = launch_mode(plan->mode, slot.d_table, L.n_large_descs, L.n_small_descs, log2k, plan->opt, s, found_inf, stream);
+    rc = launch_mode(plan->mode, slot.d_table, L, plan->opt, s, found_inf, stream);
     if (rc) return rc;
     return mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
 }
@@ -536,6 +569,7 @@ struct GradPlan {
     int64_t max_large_chunk = kMaxLargeChunk;
     int64_t unaligned_vectors = 1;
     int64_t align_heads = 1;
+    int64_t mid_tiles = 16;
     bool lazy_events = false;
     int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
     std::vector<FsGradTensor> rows;
@@ -561,9 +595,11 @@ int64_t grad_head_elems(const FsGradTensor& r, int elem_size, int64_t align_head
     return (int64_t)(((1024 - (a & 1023u)) & 1023u) / (uintptr_t)elem_size);
 }
 
-Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk, int64_t align_heads) {
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk, int64_t align_heads,
+                   int64_t mid_tiles) {
     Layout L;
     L.tile_elems = grad_tile_elems(dtype, items);
+    L.mid_chunk_elems = mid_chunk_for(L.tile_elems, mid_tiles);
     const int esz = grad_elem_size(dtype);
     int64_t min_large = 0;
     for (int64_t t = 0; t < n; ++t) {
@@ -572,11 +608,12 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
         if (numel == 0) { L.n_empty += 1; continue; }
         const int64_t head = grad_head_elems(grads[t], esz, align_heads), body = numel - head;
         (aligned_to(advance(grads[t].g, head, esz), 16) ? L.n_vector : L.n_scalar) += 1;
-        if (body >= kLargeThreshold) {
+        const int cls = class_of(body, L);
+        if (cls == kClassLarge) {
             L.n_large += 1;
             if (min_large == 0 || body < min_large) min_large = body;
         } else {
-            L.n_small += 1;
+            (cls == kClassMid ? L.n_mid : L.n_small) += 1;
         }
     }
     L.large_chunk_elems = std::min(max_large_chunk, std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2)))));
@@ -585,7 +622,9 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
         if (numel == 0) continue;
         const int64_t head = grad_head_elems(grads[t], esz, align_heads), body = numel - head;
         L.n_small_descs += ceil_div(head, L.tile_elems);
-        if (body >= kLargeThreshold) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        const int cls = class_of(body, L);
+        if (cls == kClassLarge) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
+        else if (cls == kClassMid) L.n_mid_descs += ceil_div(body, L.mid_chunk_elems);
         else L.n_small_descs += ceil_div(body, L.tile_elems);
     }
     return L;
@@ -604,8 +643,9 @@ void grad_plan_free(GradPlan* plan) {
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
 void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves,
-                int64_t* align_heads, int64_t* lazy_events) {
+                int64_t* align_heads, int64_t* lazy_events, int64_t* mid_tiles) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    *mid_tiles = g_opt.mid_tiles;
     *align_heads = g_opt.align_heads;
     *lazy_events = g_opt.lazy_events;
     // a pass that only reads pays for every small store it makes: 16 tiles share one partial
@@ -617,11 +657,10 @@ void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_ch
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
-    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk, plan->align_heads);
-    const int64_t k = L.large_chunk_elems / L.tile_elems;
-    const int64_t n_blocks = L.n_large_descs * k + L.n_small_descs;
+    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk, plan->align_heads, plan->mid_tiles);
+    const int64_t n_blocks = L.blocks();
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
-    const int64_t n_descs = L.n_large_descs + L.n_small_descs;
+    const int64_t n_descs = L.descs();
     TableSlot& slot = plan->slots[(plan->current + 1) % kTableSlots];
     int rc = mark_init(slot.mark);
     if (rc) return rc;
@@ -659,17 +698,18 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     }
     const int esz = grad_elem_size(plan->dtype);
     ChunkDesc* large = slot.h_table;
-    ChunkDesc* small = slot.h_table + L.n_large_descs;
+    ChunkDesc* mid = large + L.n_large_descs;
+    ChunkDesc* small = mid + L.n_mid_descs;
     for (int64_t t = 0; t < n; ++t) {
         const FsGradTensor& r = grads[t];
         if (r.numel == 0) continue;
         const int64_t head = grad_head_elems(r, esz, plan->align_heads);
         // pieces: the head (tile-sized descriptors), then the rest in shared chunks or tiles
-        const struct { int64_t start, count; bool large; } pieces[2] = {{0, head, false}, {head, r.numel - head, r.numel - head >= kLargeThreshold}};
+        const struct { int64_t start, count; int cls; } pieces[2] = {{0, head, kClassSmall}, {head, r.numel - head, class_of(r.numel - head, L)}};
         for (const auto& piece : pieces) {
-            const int64_t chunk_elems = piece.large ? L.large_chunk_elems : L.tile_elems;
+            const int64_t chunk_elems = piece.cls == kClassLarge ? L.large_chunk_elems : piece.cls == kClassMid ? L.mid_chunk_elems : L.tile_elems;
             const int64_t chunks = ceil_div(piece.count, chunk_elems);
-            ChunkDesc*& out = piece.large ? large : small;
+            ChunkDesc*& out = piece.cls == kClassLarge ? large : piece.cls == kClassMid ? mid : small;
             for (int64_t c = 0; c < chunks; ++c) {
                 ChunkDesc& d = out[c];
                 std::memset(&d, 0, sizeof(d));
@@ -681,7 +721,7 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
             out += chunks;
         }
     }
-    if (large != slot.h_table + L.n_large_descs || small != slot.h_table + n_descs)
+    if (large != slot.h_table + L.n_large_descs || mid != slot.h_table + L.n_large_descs + L.n_mid_descs || small != slot.h_table + n_descs)
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(grads, grads + n);
@@ -701,9 +741,8 @@ template <typename T>
 int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, int write_back, float* found_inf, double* sum_squares,
                   float* abs_max, hipStream_t stream) {
     const Layout& L = plan->layout;
-    const int log2k = log2_exact(L.large_chunk_elems / L.tile_elems);
-    const int64_t large_blocks = L.n_large_descs << log2k;
-    const int64_t n_blocks = large_blocks + L.n_small_descs;
+    const int64_t n_blocks = L.blocks();
+    const TileMap map = tile_map(L);
     TableSlot& slot = plan->slots[plan->current];
     GradPartial* first = plan->d_partials;
     GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
@@ -717,8 +756,7 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     const int64_t n_groups = ceil_div(n_blocks, waves);
 #define FS_GRAD_LAUNCH(WAVES, ITEMS)                                                                                          \
     hipLaunchKernelGGL((fsadam_grad_tiles<T, WAVES, ITEMS>), dim3((uint32_t)n_groups), dim3(64 * WAVES), lds, stream,        \
-                       slot.d_table, (uint32_t)log2k, (uint32_t)large_blocks, (uint32_t)L.n_large_descs, (uint32_t)n_blocks, \
-                       inv_scale, inv_scale_dev, write_back, first)
+                       slot.d_table, map, (uint32_t)n_blocks, inv_scale, inv_scale_dev, write_back, first)
 #define FS_GRAD_ITEMS(WAVES)                          \
     do {                                              \
         if (plan->items == 2) FS_GRAD_LAUNCH(WAVES, 2);      \
@@ -773,7 +811,8 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
 
 bool same_options(const Options& a, const Options& b) {
     return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap &&
-           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors && a.align_heads == b.align_heads;
+           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors && a.align_heads == b.align_heads &&
+           a.mid_tiles == b.mid_tiles;
 }
 
 }  // namespace
@@ -818,6 +857,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "align_heads") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "align_heads must be 0 or 1");
         g_opt.align_heads = value;
+    } else if (k == "mid_tiles") {
+        if (value < 0 || value > 64 || (value & (value - 1)) != 0) return fail(FSADAM_EINVAL, "mid_tiles must be 0 or a power of two up to 64");
+        g_opt.mid_tiles = value;
     } else if (k == "lazy_events") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "lazy_events must be 0 or 1");
         g_opt.lazy_events = value;
@@ -852,6 +894,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
     else if (k == "align_heads") *value = g_opt.align_heads;
     else if (k == "lazy_events") *value = g_opt.lazy_events;
+    else if (k == "mid_tiles") *value = g_opt.mid_tiles;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
     else if (k == "grad_waves") *value = g_opt.grad_waves;
@@ -877,11 +920,15 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
     out->n_empty_tensors = L.n_empty;
     out->n_large_descriptors = L.n_large_descs;
     out->n_small_descriptors = L.n_small_descs;
-    out->grid_large = L.n_large_descs * (L.large_chunk_elems / L.tile_elems);
+    out->grid_large = L.large_blocks();
     out->grid_small = L.n_small_descs;
+    out->mid_chunk_elems = L.mid_chunk_elems;
+    out->n_mid_tensors = L.n_mid;
+    out->n_mid_descriptors = L.n_mid_descs;
+    out->grid_mid = L.mid_blocks();
     for (int64_t t = 0; t < n_tensors; ++t) {
         const int64_t head = tensors[t].numel > 0 ? head_elems(tensors[t], precision_mode, opt) : 0;
-        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (tensors[t].numel - head >= kLargeThreshold ? 2 : 1);
+        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (uint8_t)class_of(tensors[t].numel - head, L);
         if (vector_ok) vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode, head)) ? 1 : 0;
     }
     return FSADAM_OK;
@@ -943,11 +990,11 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
     out->total_elems = L.total_elems;
     out->tile_elems = L.tile_elems;
     out->large_chunk_elems = L.large_chunk_elems;
-    out->n_descriptors = L.n_large_descs + L.n_small_descs;
+    out->n_descriptors = L.descs();
     out->n_vector_tensors = L.n_vector;
     out->n_scalar_tensors = L.n_scalar;
-    out->n_launches = (L.n_large_descs + L.n_small_descs) > 0 ? 1 : 0;
-    out->grid = L.tile_elems ? L.n_large_descs * (L.large_chunk_elems / L.tile_elems) + L.n_small_descs : 0;
+    out->n_launches = L.descs() > 0 ? 1 : 0;
+    out->grid = L.blocks();
     out->block = plan->opt.block;
     out->lds_throttle = plan->opt.lds_throttle;
     out->uploads = plan->uploads;
@@ -1023,15 +1070,15 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy;
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy, cur_mid;
     grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
-               &cur_waves, &cur_heads, &cur_lazy);
+               &cur_waves, &cur_heads, &cur_lazy, &cur_mid);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && c->align_heads == cur_heads && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && c->align_heads == cur_heads && c->mid_tiles == cur_mid && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -1057,6 +1104,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->max_large_chunk = cur_chunk;
         victim->unaligned_vectors = cur_unaligned;
         victim->align_heads = cur_heads;
+        victim->mid_tiles = cur_mid;
         victim->lazy_events = cur_lazy != 0;
         victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);

@@ -29,6 +29,32 @@ struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points a
 };
 static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");
 
+// Where the tiles of a launch find their descriptors.  Three classes of descriptors, stored one behind
+// the other: large tensors share one among 2^log2_large tiles, middle-sized ones among 2^log2_mid
+// tiles, and every tile behind those has a descriptor of its own (small tensors, heads).  A shared
+// descriptor keeps the table short (it is sent again whenever a pointer of the list moves) and lets
+// neighbouring workgroups fetch the same 64 bytes; its last tiles may lie past the end of the tensor
+// and return at once.
+struct TileMap {
+    uint32_t log2_large, n_large_blocks, n_large_descs;
+    uint32_t log2_mid, n_mid_blocks, n_mid_descs;
+};
+// descriptor index and first element (within the descriptor's chunk) of tile `block`; all operands are
+// uniform, so this is scalar arithmetic
+__device__ __forceinline__ void locate_tile(const TileMap& map, uint32_t block, uint32_t tile_elems, uint32_t& chunk, uint32_t& off) {
+    if (block < map.n_large_blocks) {
+        chunk = block >> map.log2_large;
+        off = (block & ((1u << map.log2_large) - 1u)) * tile_elems;
+    } else if (block - map.n_large_blocks < map.n_mid_blocks) {
+        const uint32_t b = block - map.n_large_blocks;
+        chunk = map.n_large_descs + (b >> map.log2_mid);
+        off = (b & ((1u << map.log2_mid) - 1u)) * tile_elems;
+    } else {
+        chunk = map.n_large_descs + map.n_mid_descs + (block - map.n_large_blocks - map.n_mid_blocks);
+        off = 0u;
+    }
+}
+
 struct StepScalars {
     const float* grad_scale_dev;  // when not NULL the kernel reads the gradient scale here instead of grad_scale
     float b1, b2, one_minus_b1, one_minus_b2;

@@ -148,8 +148,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint
 // bandwidth; with 16 waves per workgroup the cost is gone.  `n_tiles`: tiles really there (the last
 // workgroup may have fewer than WAVES).
 template <typename T, int WAVES, int ITEMS>
-__global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, uint32_t log2k, uint32_t n_large_blocks,
-                                                                uint32_t n_large_descs, uint32_t n_tiles, float inv_scale_value,
+__global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, TileMap map, uint32_t n_tiles, float inv_scale_value,
                                                                 const float* __restrict__ inv_scale_dev, int write_back,
                                                                 GradPartial* __restrict__ partials) {
     constexpr int BLOCK = 64;
@@ -166,9 +165,8 @@ __global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc*
     GradAcc acc;
     bool any = false;  // uniform within the wave
     if (block < n_tiles) {
-        const bool large = block < n_large_blocks;  // uniform: scalar selects
-        const uint32_t chunk = large ? block >> log2k : n_large_descs + (block - n_large_blocks);
-        const uint32_t off = large ? (block & ((1u << log2k) - 1u)) * kTile : 0u;
+        uint32_t chunk, off;
+        locate_tile(map, block, kTile, chunk, off);
         typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
         const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
             (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);

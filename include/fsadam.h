@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FSADAM_ABI_VERSION 1
+#define FSADAM_ABI_VERSION 2
 
 /* Precision modes = the four dtype combinations the reference dispatches on
  * (fairscale/clib/fused_adam_cuda/fused_adam_cuda_kernel.cu:172-256; Python enum
@@ -86,12 +86,16 @@ typedef struct FsAdamLayout {
     int64_t tile_elems;
     int64_t large_chunk_elems;
     int64_t n_large_tensors;     /* numel >= 131072: descriptors shared by large_chunk_elems/tile_elems tiles */
-    int64_t n_small_tensors;     /* one descriptor per tile                                                   */
+    int64_t n_small_tensors;     /* under mid_chunk_elems: one descriptor per tile                            */
     int64_t n_empty_tensors;     /* numel == 0: skipped                                                       */
     int64_t n_large_descriptors;
     int64_t n_small_descriptors;
-    int64_t grid_large;          /* workgroups of the large-tensor launch (some past a tensor's end: they exit) */
-    int64_t grid_small;          /* workgroups of the small-tensor launch                                      */
+    int64_t grid_large;          /* workgroups of the large tensors (some past a tensor's end: they exit)       */
+    int64_t grid_small;          /* workgroups with a descriptor of their own                                  */
+    int64_t mid_chunk_elems;     /* elements per shared descriptor of a middle-sized tensor; 0: no such class   */
+    int64_t n_mid_tensors;       /* mid_chunk_elems <= numel < 131072                                          */
+    int64_t n_mid_descriptors;
+    int64_t grid_mid;            /* workgroups of the middle-sized tensors                                     */
 } FsAdamLayout;
 
 /* ---- library ---- */
@@ -127,6 +131,10 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   into a flat buffer) gives its first elements, at most 511, to a short descriptor of their own, so
  *                   that every tile behind them starts on line boundaries (see fsadam_head_elems); 0: tiles start
  *                   at element 0 wherever that is (lists of packed views measured 20 % slower)
+ *   "mid_tiles"     tiles that share one descriptor of a middle-sized tensor (one of at least mid_tiles tiles and
+ *                   under 131072 elements): 0 (every such tile has its own descriptor) or a power of two up to 64
+ *                   (default 16).  Shared descriptors make the table of a many-tensor list 10x shorter, which is
+ *                   what is sent again when a pointer of the list moves
  *   "lazy_events"   0 (default): an event is recorded behind every step (and gradient pass); it is what the library
  *                   waits for before it overwrites a table a step may still read, and what orders a call on
  *                   another stream behind the one before.  1: the event is only recorded when one of those needs
@@ -188,7 +196,7 @@ int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float be
                                float* found_inf_dev, void* hip_stream);
 
 /* Host-only planning (no device needed): how the list would be laid out under the current options.
- * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large.  vector_ok[n_tensors] (may be
+ * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large, 3 middle-sized.  vector_ok[n_tensors] (may be
  * NULL): 1 = every stream aligned to its 64/128-bit vector. */
 int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
                   uint8_t* tensor_class, uint8_t* vector_ok);

@@ -75,7 +75,7 @@ def test_step_size_is_bit_identical_to_the_oracle(oracle):
 
 def test_options_roundtrip_and_validation():
     old = {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "grad_waves", "grad_items",
-                                                "grad_lds_throttle", "unaligned_vectors", "align_heads", "lazy_events")}
+                                                "grad_lds_throttle", "unaligned_vectors", "align_heads", "lazy_events", "mid_tiles")}
     try:
         _cabi.set_option("block", 128)
         _cabi.set_option("groups", 2)
@@ -86,7 +86,7 @@ def test_options_roundtrip_and_validation():
                 _cabi.set_option(flag, value)
                 assert _cabi.get_option(flag) == value
         for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", -1), ("max_large_chunk", 5000), ("max_large_chunk", 2048), ("grad_waves", 3), ("grad_items", 5), ("unaligned_vectors", 2),
-                          ("align_heads", 2), ("lazy_events", -1), ("no_such_option", 1)):
+                          ("align_heads", 2), ("lazy_events", -1), ("mid_tiles", 3), ("mid_tiles", 128), ("no_such_option", 1)):
             with pytest.raises(_cabi.FsAdamError):
                 _cabi.set_option(name, bad)
     finally:
@@ -106,10 +106,11 @@ def layout(tensors, mode):
 def test_layout_classes_and_descriptor_counts():
     A = 0x7000_0000_0000  # fake, 2 MiB-aligned device addresses: never dereferenced on the host
     t = lambda n, off=0: (A + off, A + (1 << 32), A + (2 << 32), A + (3 << 32) + off, 0, n)  # noqa: E731
-    old = {k: _cabi.get_option(k) for k in ("block", "groups")}
+    old = {k: _cabi.get_option(k) for k in ("block", "groups", "mid_tiles")}
     try:
         _cabi.set_option("block", 64)
         _cabi.set_option("groups", 1)
+        _cabi.set_option("mid_tiles", 0)  # two classes: shared descriptors from 131072 elements, one per tile below
         lay, cls, vec = layout([t(0), t(1), t(255), t(256), t(257), t(131071), t(131072), t(131073), t(1 << 20)], _cabi.FULL_PRECISION)
         assert lay["tile_elems"] == 256  # 64 lanes x 4 fp32
         assert cls == [0, 1, 1, 1, 1, 1, 2, 2, 2]
@@ -120,7 +121,19 @@ def test_layout_classes_and_descriptor_counts():
         assert lay["n_large_descriptors"] == 2 + 3 + 16
         assert lay["grid_large"] == lay["n_large_descriptors"] * (65536 // 256)
         assert lay["grid_small"] == lay["n_small_descriptors"]
+        assert (lay["mid_chunk_elems"], lay["n_mid_tensors"], lay["n_mid_descriptors"], lay["grid_mid"]) == (0, 0, 0, 0)
         assert vec == [0, 1, 1, 1, 1, 1, 1, 1, 1]
+        # three classes (the default): 16 tiles = 4096 elements share a descriptor from 4096 elements on
+        _cabi.set_option("mid_tiles", 16)
+        lay, cls, _ = layout([t(0), t(1), t(4095), t(4096), t(4097), t(131071), t(131072)], _cabi.FULL_PRECISION)
+        assert cls == [0, 1, 1, 3, 3, 3, 2] and lay["mid_chunk_elems"] == 4096
+        assert (lay["n_small_tensors"], lay["n_mid_tensors"], lay["n_large_tensors"]) == (2, 3, 1)
+        assert lay["n_small_descriptors"] == 1 + 16 and lay["n_mid_descriptors"] == 1 + 2 + 32 and lay["n_large_descriptors"] == 2
+        assert lay["grid_mid"] == 35 * 16 and lay["grid_small"] == 17 and lay["grid_large"] == 2 * 256
+        _cabi.set_option("mid_tiles", 64)  # 16384 elements
+        lay, cls, _ = layout([t(16383), t(16384), t(100000)], _cabi.FULL_PRECISION)
+        assert cls == [1, 3, 3] and lay["mid_chunk_elems"] == 16384 and lay["n_mid_descriptors"] == 1 + 7 and lay["grid_mid"] == 8 * 64
+        _cabi.set_option("mid_tiles", 0)
         # one 1.63e9-element tensor: chunk capped at 2^24, 98 descriptors
         lay, cls, _ = layout([t(1_630_000_000)], _cabi.MEMORY_EFFICIENT_MIXED_PRECISION)
         assert lay["large_chunk_elems"] == 1 << 24 and lay["n_large_descriptors"] == 98 and cls == [2]
@@ -134,6 +147,15 @@ def test_layout_classes_and_descriptor_counts():
     finally:
         for k, v in old.items():
             _cabi.set_option(k, v)
+
+
+@pytest.fixture
+def two_classes():
+    """No middle class for one test: every tile of a tensor under 131072 elements has its own descriptor."""
+    old = _cabi.get_option("mid_tiles")
+    _cabi.set_option("mid_tiles", 0)
+    yield
+    _cabi.set_option("mid_tiles", old)
 
 
 def head_of(t, mode):
@@ -214,7 +236,7 @@ def test_no_other_head_would_align_better():
         assert (cost(got), got) == (cost(best), best), (case, mode, [hex(s[0]) for s in streams], got, best)
 
 
-def test_layout_counts_heads_among_the_small_descriptors():
+def test_layout_counts_heads_among_the_small_descriptors(two_classes):
     A = 0x7000_0000_0000
     t = lambda n, off: (A + off, A + (1 << 34) + off, A + (2 << 34) + off, A + (3 << 34) + off, 0, n)  # noqa: E731
     # 100 elements short of a 1 KiB boundary: head 100, then exactly two shared chunks
@@ -246,13 +268,14 @@ def test_layout_matches_a_python_model_on_drawn_lists():
 
     rng = random.Random(42)
     A = 0x7000_0000_0000
-    names = ("block", "groups", "max_large_chunk")
+    names = ("block", "groups", "max_large_chunk", "mid_tiles")
     old = {k: _cabi.get_option(k) for k in names}
     try:
-        for _ in range(60):
+        for _ in range(120):
             block, groups = rng.choice([64, 128, 256]), rng.choice([1, 2])
             cap = rng.choice([1 << 24, 1 << 16, 1 << 14, 4096])
-            for k, v in zip(names, (block, groups, cap)):
+            mid_tiles = rng.choice([0, 1, 2, 16, 16, 64])
+            for k, v in zip(names, (block, groups, cap, mid_tiles)):
                 _cabi.set_option(k, v)
             mode = rng.choice([_cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16])
             sizes = [rng.choice([0, 1, rng.randrange(2, 5000), rng.randrange(5000, 131072), 131072, rng.randrange(131072, 1 << 22),
@@ -264,14 +287,19 @@ def test_layout_matches_a_python_model_on_drawn_lists():
                 chunk = 1 << ((min(large) // 2).bit_length() - 1)
             chunk = min(cap, max(65536, min(1 << 24, chunk)))
             want_large = sum(-(-n // chunk) for n in large)
-            want_small = sum(-(-n // tile) for n in sizes if 0 < n < 131072)
+            # a middle class only for 2..64 tiles per descriptor and chunks of at most half the large threshold
+            mid_chunk = tile * mid_tiles if mid_tiles > 1 and 2 * tile * mid_tiles <= 131072 else 0
+            is_mid = lambda n: mid_chunk and mid_chunk <= n < 131072  # noqa: E731
+            want_mid = sum(-(-n // mid_chunk) for n in sizes if is_mid(n))
+            want_small = sum(-(-n // tile) for n in sizes if 0 < n < 131072 and not is_mid(n))
             rows_ = [(A, A + (1 << 40), A + (2 << 40), A + (3 << 40), A + (4 << 40) if mode == _cabi.MIXED_PRECISION else 0, n) for n in sizes]
             lay, cls, _ = layout(rows_, mode)
             what = f"block {block} groups {groups} cap {cap} mode {mode} sizes {sizes}"
             assert lay["tile_elems"] == tile and lay["large_chunk_elems"] == chunk, what
             assert lay["n_large_descriptors"] == want_large and lay["n_small_descriptors"] == want_small, what
             assert lay["grid_large"] == want_large * (chunk // tile) and lay["grid_small"] == want_small, what
-            assert cls == [0 if n == 0 else (2 if n >= 131072 else 1) for n in sizes], what
+            assert lay["mid_chunk_elems"] == mid_chunk and lay["n_mid_descriptors"] == want_mid and lay["grid_mid"] == want_mid * mid_tiles, what
+            assert cls == [0 if n == 0 else (2 if n >= 131072 else 3 if is_mid(n) else 1) for n in sizes], what
     finally:
         for k, v in old.items():
             _cabi.set_option(k, v)

@@ -134,6 +134,25 @@ def test_every_compiled_shape_of_the_pass_matches_the_oracle(cuda_device, dtype,
             _cabi.set_option(k, v)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("mid_tiles", [0, 2, 16, 64])
+def test_descriptors_shared_by_a_few_tiles_do_not_change_the_pass(cuda_device, dtype, mid_tiles):
+    """Middle-sized gradients share a descriptor among `mid_tiles` tiles (none with 0).  Sizes around the
+    chunk boundaries that result for both dtypes and both kinds of pass."""
+    from fairscale_amd import _cabi
+
+    sizes = [1, 4095, 4096, 4097, 8191, 8192, 8193, 16384, 32767, 32768, 32769, 65535, 65536, 65537, 100000, 131071, 131072, 200001]
+    old = _cabi.get_option("mid_tiles")
+    _cabi.set_option("mid_tiles", mid_tiles)
+    try:
+        for write_back in (False, True):
+            host = host_grads(dtype, 14, sizes, scale=64.0)
+            dev, stats, want = run_both(host, cuda_device, 1 / 64, write_back, misalign=3)
+            check(host, dev, stats, want, f"mid_tiles {mid_tiles} wb {write_back}")
+    finally:
+        _cabi.set_option("mid_tiles", old)
+
+
 def test_unscale_by_an_inexact_factor_rounds_twice_on_every_path(cuda_device):
     """half(float32(float(g) * inv_scale)): the float32 rounding comes first, as in torch's kernel.  Many
     tensors just below one tile (element-wise path) plus a large one (vector path), enough elements for

@@ -118,8 +118,10 @@ def test_c1_full_precision_flat_2pow20(oracle, cuda_device):
 def test_modes_edge_sizes(oracle, cuda_device, mode, eps_mode, bias_correction):
     """Every dtype combination x eps placement x bias correction over sizes around every boundary
     the kernel has: vector width (4/8), tile (256..4096), the reference's 65536 chunk, the
-    small/large tensor threshold (131072) and a large tensor that ends just into a shared chunk."""
-    sizes = [1, 2, 3, 4, 5, 7, 8, 9, 15, 17, 255, 256, 257, 511, 513, 1023, 1025, 2047, 2048, 2049, 4095, 4097, 16383, 16384, 16385,
+    descriptors shared by 16 tiles (from 4096 elements, 8192 in PURE_FP16), the small/large tensor threshold
+    (131072) and a large tensor that ends just into a shared chunk."""
+    sizes = [1, 2, 3, 4, 5, 7, 8, 9, 15, 17, 255, 256, 257, 511, 513, 1023, 1025, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193, 12289,
+             16383, 16384, 16385,
              32769, 65535, 65536, 65537, 100003, 131071, 131072, 131073, 196611, 262144 + 5]
     hyper = dict(DEFAULT, eps_mode=eps_mode, bias_correction=bias_correction, decay=0.01)
     gs = 1.0 if mode == FULL else 1024.0
@@ -276,7 +278,7 @@ def options():
     """Set tuning options for one test and put the defaults back afterwards."""
     from fairscale_amd import _cabi
 
-    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events")
+    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events", "mid_tiles")
     old = {k: _cabi.get_option(k) for k in names}
 
     def set_many(**kw):
@@ -301,11 +303,12 @@ def test_every_compiled_tile_shape_matches_the_oracle(oracle, cuda_device, optio
 
 
 @pytest.mark.parametrize("setting", [dict(xcd_remap=1), dict(xcd_remap=7), dict(xcd_remap=1 << 20), dict(lds_throttle=0),
-                                     dict(lds_throttle=65536), dict(max_large_chunk=4096), dict(max_large_chunk=65536, block=256, groups=2)])
+                                     dict(lds_throttle=65536), dict(max_large_chunk=4096), dict(max_large_chunk=65536, block=256, groups=2),
+                                     dict(mid_tiles=0), dict(mid_tiles=2), dict(mid_tiles=64), dict(mid_tiles=4, block=128, xcd_remap=3)])
 def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, options, setting):
     options(**setting)
     for mode in (MEMEFF, PURE16):
-        run_case(oracle, cuda_device, mode, [5, 4099, 40000, 140001, 524288 + 17], 2, 4900 + mode, DEFAULT, grad_scale=8.0,
+        run_case(oracle, cuda_device, mode, [5, 4099, 40000, 16384, 131071, 140001, 524288 + 17], 2, 4900 + mode, DEFAULT, grad_scale=8.0,
                  optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
