@@ -388,7 +388,10 @@ int refuse_capture(hipStream_t stream) {
 }
 
 void plan_release_buffers(FsAdamPlan* plan) {
-    for (TableSlot& slot : plan->slots) slot_release(slot);
+    for (TableSlot& slot : plan->slots) {
+        slot_release(slot);
+        mark_destroy(slot.mark);  // an event belongs to the device it was created on
+    }
     plan->current = -1;
 }
 
@@ -1004,7 +1007,6 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
 int fsadam_plan_destroy(FsAdamPlan* plan) {
     if (!plan) return FSADAM_OK;
     plan_release_buffers(plan);
-    for (TableSlot& slot : plan->slots) mark_destroy(slot.mark);
     delete plan;
     return FSADAM_OK;
 }
