@@ -83,6 +83,7 @@ struct Options {
     int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
     int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
     int64_t mid_tiles = 16;         // tiles that share a descriptor of a middle-sized tensor (a power of two up to 64; 0 = no such class)
+    int64_t upload_stream = 1;      // 1: tables are copied to the device on a stream of the library's own
     int64_t lazy_events = 0;        // 1: events behind steps are recorded only when needed (streams must outlive the plan)
     int64_t align_heads = 1;        // 1: a tensor whose streams start off a cache line gives up a short head so that the rest starts on one
 };
@@ -304,12 +305,14 @@ struct TableSlot {
     ChunkDesc* d_table = nullptr;
     ChunkDesc* h_table = nullptr;  // pinned
     UseMark mark;
+    hipEvent_t uploaded = nullptr;  // the copy of h_table into d_table, when it went over the library's own stream
 };
 constexpr int kTableSlots = 3;
 
 struct FsAdamPlan {
     int mode = 0;
     int device = -1;
+    hipStream_t upload_stream = nullptr;  // the library's own, for tables (see upload_table)
     Options opt;
     Layout layout;
     std::vector<FsAdamTensor> rows;  // what the current table was built from
@@ -367,6 +370,31 @@ void mark_destroy(UseMark& m) {
     m = UseMark();
 }
 
+// A new table is copied to the device on a stream of the library's own and the caller's stream only waits
+// for that copy's event: the copy (1.4 MB for a 4096-tensor list, 60 us) then runs while the step before
+// is still busy on the caller's stream instead of between the two steps.  `own_stream` = 0 (option
+// "upload_stream") puts the copy on the caller's stream.
+int upload_table(hipStream_t* own, bool use_own, TableSlot& slot, int64_t n_descs, hipStream_t stream) {
+    if (n_descs <= 0) return FSADAM_OK;
+    const size_t bytes = (size_t)n_descs * sizeof(ChunkDesc);
+    if (!use_own) {
+        FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, bytes, hipMemcpyHostToDevice, stream));
+        return FSADAM_OK;
+    }
+    if (!*own) FS_HIP(hipStreamCreateWithFlags(own, hipStreamNonBlocking));
+    if (!slot.uploaded) FS_HIP(hipEventCreateWithFlags(&slot.uploaded, hipEventDisableTiming));
+    FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, bytes, hipMemcpyHostToDevice, *own));
+    FS_HIP(hipEventRecord(slot.uploaded, *own));
+    FS_HIP(hipStreamWaitEvent(stream, slot.uploaded, 0));
+    return FSADAM_OK;
+}
+void upload_stream_destroy(hipStream_t* own) {
+    if (!*own) return;
+    (void)hipStreamSynchronize(*own);
+    (void)hipStreamDestroy(*own);
+    *own = nullptr;
+}
+
 void slot_release(TableSlot& slot) {
     (void)mark_wait(slot.mark);
     if (slot.d_table) (void)hipFree(slot.d_table);
@@ -387,11 +415,17 @@ int refuse_capture(hipStream_t stream) {
     return FSADAM_OK;
 }
 
+// events and streams belong to the device they were created on: they go with the buffers
+void slot_destroy(TableSlot& slot) {
+    slot_release(slot);
+    mark_destroy(slot.mark);
+    if (slot.uploaded) (void)hipEventDestroy(slot.uploaded);
+    slot.uploaded = nullptr;
+}
+
 void plan_release_buffers(FsAdamPlan* plan) {
-    for (TableSlot& slot : plan->slots) {
-        slot_release(slot);
-        mark_destroy(slot.mark);  // an event belongs to the device it was created on
-    }
+    for (TableSlot& slot : plan->slots) slot_destroy(slot);
+    upload_stream_destroy(&plan->upload_stream);
     plan->current = -1;
 }
 
@@ -512,8 +546,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(tensors, tensors + n);
-    if (n_descs > 0)
-        FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
+    rc = upload_table(&plan->upload_stream, plan->opt.upload_stream != 0, slot, n_descs, stream);
+    if (rc) return rc;
     rc = mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
     if (rc) return rc;
     // the steps that used the table this one replaces are all enqueued: their slot's event can be taken now
@@ -574,6 +608,8 @@ struct GradPlan {
     int64_t align_heads = 1;
     int64_t mid_tiles = 16;
     bool lazy_events = false;
+    bool own_upload_stream = true;
+    hipStream_t upload_stream = nullptr;
     int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
     std::vector<FsGradTensor> rows;
     Layout layout;
@@ -635,10 +671,8 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
 
 void grad_plan_free(GradPlan* plan) {
     mark_destroy(plan->partials_mark);
-    for (TableSlot& slot : plan->slots) {
-        slot_release(slot);
-        mark_destroy(slot.mark);
-    }
+    for (TableSlot& slot : plan->slots) slot_destroy(slot);
+    upload_stream_destroy(&plan->upload_stream);
     if (plan->d_partials) (void)hipFree(plan->d_partials);
     delete plan;
 }
@@ -646,8 +680,9 @@ void grad_plan_free(GradPlan* plan) {
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
 void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves,
-                int64_t* align_heads, int64_t* lazy_events, int64_t* mid_tiles) {
+                int64_t* align_heads, int64_t* lazy_events, int64_t* mid_tiles, int64_t* upload_stream) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    *upload_stream = g_opt.upload_stream;
     *mid_tiles = g_opt.mid_tiles;
     *align_heads = g_opt.align_heads;
     *lazy_events = g_opt.lazy_events;
@@ -728,8 +763,8 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(grads, grads + n);
-    if (n_descs > 0)
-        FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc), hipMemcpyHostToDevice, stream));
+    rc = upload_table(&plan->upload_stream, plan->own_upload_stream, slot, n_descs, stream);
+    if (rc) return rc;
     rc = mark_use(slot.mark, stream, plan->lazy_events);
     if (rc) return rc;
     if (plan->current >= 0) {
@@ -863,6 +898,9 @@ int fsadam_set_option(const char* name, int64_t value) {
     } else if (k == "mid_tiles") {
         if (value < 0 || value > 64 || (value & (value - 1)) != 0) return fail(FSADAM_EINVAL, "mid_tiles must be 0 or a power of two up to 64");
         g_opt.mid_tiles = value;
+    } else if (k == "upload_stream") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "upload_stream must be 0 or 1");
+        g_opt.upload_stream = value;
     } else if (k == "lazy_events") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "lazy_events must be 0 or 1");
         g_opt.lazy_events = value;
@@ -897,6 +935,7 @@ int fsadam_get_option(const char* name, int64_t* value) {
     else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
     else if (k == "align_heads") *value = g_opt.align_heads;
     else if (k == "lazy_events") *value = g_opt.lazy_events;
+    else if (k == "upload_stream") *value = g_opt.upload_stream;
     else if (k == "mid_tiles") *value = g_opt.mid_tiles;
     else if (k == "grad_items") *value = g_opt.grad_items;
     else if (k == "grad_lds_throttle") *value = g_opt.grad_lds_throttle;
@@ -1072,9 +1111,9 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy, cur_mid;
+    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy, cur_mid, cur_upload;
     grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
-               &cur_waves, &cur_heads, &cur_lazy, &cur_mid);
+               &cur_waves, &cur_heads, &cur_lazy, &cur_mid, &cur_upload);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
@@ -1107,6 +1146,7 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         victim->unaligned_vectors = cur_unaligned;
         victim->align_heads = cur_heads;
         victim->mid_tiles = cur_mid;
+        victim->own_upload_stream = cur_upload != 0;
         victim->lazy_events = cur_lazy != 0;
         victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);

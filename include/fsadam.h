@@ -135,6 +135,9 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   under 131072 elements): 0 (every such tile has its own descriptor) or a power of two up to 64
  *                   (default 16).  Shared descriptors make the table of a many-tensor list 10x shorter, which is
  *                   what is sent again when a pointer of the list moves
+ *   "upload_stream" 1 (default): a new descriptor table is copied to the device on a stream the library owns,
+ *                   and the caller's stream waits for that copy's event, so the copy overlaps the step still
+ *                   running on the caller's stream; 0: the copy is enqueued on the caller's stream
  *   "lazy_events"   0 (default): an event is recorded behind every step (and gradient pass); it is what the library
  *                   waits for before it overwrites a table a step may still read, and what orders a call on
  *                   another stream behind the one before.  1: the event is only recorded when one of those needs

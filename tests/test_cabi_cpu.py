@@ -75,18 +75,18 @@ def test_step_size_is_bit_identical_to_the_oracle(oracle):
 
 def test_options_roundtrip_and_validation():
     old = {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "grad_waves", "grad_items",
-                                                "grad_lds_throttle", "unaligned_vectors", "align_heads", "lazy_events", "mid_tiles")}
+                                                "grad_lds_throttle", "unaligned_vectors", "align_heads", "lazy_events", "mid_tiles", "upload_stream")}
     try:
         _cabi.set_option("block", 128)
         _cabi.set_option("groups", 2)
         _cabi.set_option("lds_throttle", 20480)
         assert (_cabi.get_option("block"), _cabi.get_option("groups"), _cabi.get_option("lds_throttle")) == (128, 2, 20480)
-        for flag in ("align_heads", "lazy_events"):
+        for flag in ("align_heads", "lazy_events", "upload_stream"):
             for value in (0, 1):
                 _cabi.set_option(flag, value)
                 assert _cabi.get_option(flag) == value
         for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", -1), ("max_large_chunk", 5000), ("max_large_chunk", 2048), ("grad_waves", 3), ("grad_items", 5), ("unaligned_vectors", 2),
-                          ("align_heads", 2), ("lazy_events", -1), ("mid_tiles", 3), ("mid_tiles", 128), ("no_such_option", 1)):
+                          ("align_heads", 2), ("lazy_events", -1), ("mid_tiles", 3), ("mid_tiles", 128), ("upload_stream", 2), ("no_such_option", 1)):
             with pytest.raises(_cabi.FsAdamError):
                 _cabi.set_option(name, bad)
     finally:

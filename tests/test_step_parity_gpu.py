@@ -278,7 +278,7 @@ def options():
     """Set tuning options for one test and put the defaults back afterwards."""
     from fairscale_amd import _cabi
 
-    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events", "mid_tiles")
+    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events", "mid_tiles", "upload_stream")
     old = {k: _cabi.get_option(k) for k in names}
 
     def set_many(**kw):
@@ -313,15 +313,17 @@ def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, opti
 
 
 @pytest.mark.parametrize("lazy_events", [0, 1])
-def test_event_bookkeeping_eager_and_lazy(oracle, cuda_device, options, lazy_events):
+@pytest.mark.parametrize("upload_stream", [1, 0])
+def test_event_bookkeeping_eager_and_lazy(oracle, cuda_device, options, lazy_events, upload_stream):
     """The event behind a step is what protects a table that may still be read and what orders a step on
     another stream behind the one before.  Recorded behind every step (the library's default) or only when
     needed (what this package switches on, torch's streams being immortal), the results are the same:
     steps hopping between three streams without any synchronisation by the caller, with the gradient
-    pointers moving every step (a new table every step, the ring of slots wrapping around)."""
+    pointers moving every step (a new table every step, the ring of slots wrapping around).  The tables
+    travel on a stream of the library's own (default) or on the caller's."""
     from fairscale_amd import fused_adam_hip
 
-    options(lazy_events=lazy_events)
+    options(lazy_events=lazy_events, upload_stream=upload_stream)
     host = C.Tensors(FULL, [5, 4099, 140001, 70000], 5100)
     dev = GpuList(host, cuda_device)
     streams = [torch.cuda.Stream(cuda_device) for _ in range(3)]
@@ -337,7 +339,7 @@ def test_event_bookkeeping_eager_and_lazy(oracle, cuda_device, options, lazy_eve
             plan.step([dev.p, dev.m, dev.v, g], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, dev.found_inf, step, 1, 1, 0.0)
         oracle_step(oracle, host, grads, flag, **dict(DEFAULT, step=step))
     torch.cuda.synchronize(cuda_device)
-    compare(host, dev, f"lazy_events={lazy_events}")
+    compare(host, dev, f"lazy_events={lazy_events} upload_stream={upload_stream}")
     assert plan.info()["uploads"] == 12
     plan.close()
 
