@@ -174,8 +174,9 @@ def adam(chunk_size: int, noop_flag: Optional[torch.Tensor], tensor_lists: List[
         raise RuntimeError("found_inf must live on the tensors' device")
     L = _cabi.lib()
     with _on_device(device):
-        _cabi.check(L.fsadam_step(_rows_ptr(rows), rows.shape[0], precision, lr, beta1, beta2, eps, grad_scale,
-                                  optim_scale, decay, int(step), int(mode), int(bias_correction),
+        # float(): pybind narrows whatever has __float__ (numpy scalars, one-element tensors); so does this
+        _cabi.check(L.fsadam_step(_rows_ptr(rows), rows.shape[0], precision, float(lr), float(beta1), float(beta2), float(eps),
+                                  float(grad_scale), float(optim_scale), float(decay), int(step), int(mode), int(bias_correction),
                                   found_inf.data_ptr(), _stream_handle(device)))
 
 
@@ -235,6 +236,8 @@ class TensorListPlan:
         scale_on_device = isinstance(grad_scale, torch.Tensor)
         if scale_on_device and (grad_scale.dtype != torch.float32 or grad_scale.numel() != 1 or grad_scale.device != self.device):
             raise RuntimeError("a tensor scale must be float32 with one element on the parameters' device")
+        # a scheduler may leave a numpy scalar or a one-element tensor in the group: float() as pybind would
+        lr, beta1, beta2, eps, optim_scale, decay = float(lr), float(beta1), float(beta2), float(eps), float(optim_scale), float(decay)
         with _on_device(self.device):
             stream = _stream_handle(self.device)
             if changed or self._dirty:
@@ -245,7 +248,7 @@ class TensorListPlan:
                 _cabi.check(L.fsadam_plan_step_dev_scale(self._handle, lr, beta1, beta2, eps, grad_scale.data_ptr(), optim_scale,
                                                          decay, int(step), int(eps_mode), int(bias_correction), flag, stream))
             else:
-                _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, grad_scale, optim_scale, decay,
+                _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, float(grad_scale), optim_scale, decay,
                                                int(step), int(eps_mode), int(bias_correction), flag, stream))
 
     def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,

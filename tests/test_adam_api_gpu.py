@@ -520,6 +520,24 @@ def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_
             assert torch.equal(fresh.state[q][key], opts[1].state[q][key])
 
 
+def test_hyperparameters_left_as_numpy_scalars_or_tensors_are_accepted(api, cuda_device):
+    """A scheduler may leave ``np.float32`` or a one-element tensor in ``group["lr"]``; the reference's binding
+    converts anything with ``__float__`` (fused_adam_cuda.cpp:4-8), and the result is that of the plain float."""
+    Adam, _, _ = api
+    outs = []
+    for lr, wd in ((1e-2, 0.01), (np.float32(1e-2), np.float64(0.01)), (torch.tensor(1e-2), torch.tensor(0.01, dtype=torch.float64))):
+        params = _random_problem("FULL_PRECISION", cuda_device)
+        opt = Adam(params, lr=1e-2, weight_decay=0.01)
+        opt.param_groups[0]["lr"], opt.param_groups[0]["weight_decay"] = lr, wd
+        for step in range(1, 4):
+            _set_grads(params, step)
+            opt.step()
+        outs.append([p.detach().clone() for p in params])
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert torch.equal(a, b)
+
+
 def test_list_walk_helper_is_loaded():
     from fairscale_amd import _rows
 
