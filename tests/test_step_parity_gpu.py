@@ -686,6 +686,57 @@ def test_c4_flat_shard_1p63e9_memory_efficient(oracle, cuda_device):
     _window_check(oracle, MEMEFF, before, sub, gs, [(0, cnt)], dict(DEFAULT, step=3, grad_scale=1024.0), "C4 misaligned view")
 
 
+def test_c4_size_properties_that_need_no_oracle(cuda_device):
+    """The 1.63e9-element shard again, checked through what holds at any size: the same step on the same
+    bits gives the same bits (two runs); gradients doubled together with the gradient scale change nothing
+    (a power of two moves only the exponent); the buffer stepped as one tensor or as 1000 uneven views that
+    start at odd elements (heads, shared and single descriptors, ragged ends at full scale) gives the same
+    bits; and in MIXED_PRECISION the fp16 copy is exactly half(p32) everywhere."""
+    from fairscale_amd import fused_adam_hip
+    import random
+
+    n = 1_630_000_000
+    dev = cuda_device
+    gen = torch.Generator(device=dev).manual_seed(4100)
+    p0 = (torch.randn(n, device=dev, generator=gen, dtype=torch.float32) * 0.02).half()
+    g = (torch.randn(n, device=dev, generator=gen, dtype=torch.float32) * (1e-3 * 1024)).half()
+    m0 = torch.randn(n, device=dev, generator=gen, dtype=torch.float32) * 1e-3
+    v0 = (torch.randn(n, device=dev, generator=gen, dtype=torch.float32) * 1e-3).square_()
+    flag = torch.zeros(1, device=dev)
+
+    def step(lists, scale):
+        fused_adam_hip.adam(65536, None, lists, 1e-3, 0.9, 0.999, 1e-8, scale, 1.0, flag, 7, 1, 1, 0.01)
+
+    ref = [p0.clone(), m0.clone(), v0.clone()]
+    step([[ref[0]], [ref[1]], [ref[2]], [g]], 1024.0)
+    # the same again
+    again = [p0.clone(), m0.clone(), v0.clone()]
+    step([[again[0]], [again[1]], [again[2]], [g]], 1024.0)
+    assert all(torch.equal(a, b) for a, b in zip(ref, again)), "two runs differ"
+    # doubled gradients, doubled scale (|g| stays far below the fp16 maximum)
+    again = [p0.clone(), m0.clone(), v0.clone()]
+    g2 = g * 2
+    assert torch.isfinite(g2).all()
+    step([[again[0]], [again[1]], [again[2]], [g2]], 2048.0)
+    assert all(torch.equal(a, b) for a, b in zip(ref, again)), "power-of-two scale changed the result"
+    del g2
+    # 1000 uneven views, cut at drawn (mostly odd) elements
+    rng = random.Random(4101)
+    cuts = sorted({0, n} | {rng.randrange(1, n) for _ in range(999)})
+    again = [p0.clone(), m0.clone(), v0.clone()]
+    lists = [[t[a:b] for a, b in zip(cuts[:-1], cuts[1:])] for t in (again[0], again[1], again[2], g)]
+    step(lists, 1024.0)
+    assert all(torch.equal(a, b) for a, b in zip(ref, again)), "split into views changed the result"
+    del again, lists, ref
+    torch.cuda.empty_cache()
+    # MIXED_PRECISION: fp32 master, fp16 copy out
+    p32 = p0.float()
+    p16 = torch.empty_like(p0)
+    step([[p32], [m0], [v0], [g], [p16]], 1024.0)
+    assert torch.equal(p16, p32.half())
+    assert flag.item() == 0.0
+
+
 def test_single_tensor_beyond_2_to_31_elements(oracle, cuda_device):
     """One fp16 tensor of 2^31 + 2^20 + 5 elements (PURE_FP16, 17 GB): element counts and offsets are 64-bit
     here (the reference keeps them in int, multi_tensor_apply.cuh:21,80).  Windows at the start, across
