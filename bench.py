@@ -220,14 +220,23 @@ def measure_cpu(torch, precision_name, numel, budget_s=15.0):
             "sample": f"{done} steps of the same {precision_name} math (in-place torch CPU ops, oracle/adam_torch_cpu.py) on a flat {numel}-parameter buffer, {el:.1f} s"}
 
 
+# counter summaries under profiles/ that hold "traffic = <bytes> bytes per launch" for a workload
+TRAFFIC_SUMMARIES = {"flat_shard_1630000000_MEMORY_EFFICIENT_MIXED_PRECISION": "fsadam_tiles_flat_shard_1p63e9_hbm_counters.txt"}
+
+
 def load_traffic(workload_key):
     """HBM bytes per launch from the committed counter summary, if there is one for this workload."""
-    path = os.path.join(REPO, "profiles", "hbm_traffic.json")
-    try:
-        with open(path) as fh:
-            return json.load(fh).get(workload_key, {}).get("traffic_bytes_per_launch")
-    except (OSError, ValueError):
+    import re
+
+    name = TRAFFIC_SUMMARIES.get(workload_key)
+    if name is None:
         return None
+    try:
+        with open(os.path.join(REPO, "profiles", name)) as fh:
+            found = re.search(r"traffic = (\d+) bytes per launch", fh.read())
+    except OSError:
+        return None
+    return int(found.group(1)) if found else None
 
 
 def main():
