@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import sys
 from typing import List, Optional, Sequence
 
 import numpy as np
@@ -203,6 +204,8 @@ class TensorListPlan:
                 self._handle = ctypes.c_void_p()
 
     def __del__(self):  # pragma: no cover - interpreter shutdown order is not ours to test
+        if sys.is_finalizing():
+            return  # the process is ending: nothing to give back, and the runtime underneath may be half gone
         try:
             self.close()
         except Exception:
