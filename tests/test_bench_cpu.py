@@ -1,0 +1,38 @@
+"""What can be said about bench.py without a GPU: it refuses more than one GPU with a message, its
+HBM-traffic figure comes out of the committed counter summary, and its byte counts per parameter are the
+ones the update equations imply."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    proc = subprocess.run([sys.executable, os.path.join(REPO, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                          text=True, timeout=120)
+    assert proc.returncode == 2
+    assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_traffic_figure_comes_from_the_counter_summary():
+    import bench
+
+    got = bench.load_traffic("flat_shard_1630000000_MEMORY_EFFICIENT_MIXED_PRECISION")
+    algorithmic = 22 * 1_630_000_000
+    assert isinstance(got, int) and abs(got - algorithmic) < 0.01 * algorithmic  # measured traffic = algorithmic bytes within 1 %
+    assert bench.load_traffic("some other workload") is None
+    for name in os.listdir(os.path.join(REPO, "profiles")):
+        assert name.endswith((".txt", ".md")), f"profiles/ holds text summaries only, found {name}"
+
+
+def test_bytes_per_parameter_follow_from_the_streams():
+    import bench
+
+    # reads p, m, v, g + writes p, m, v (+ the fp16 copy in MIXED_PRECISION); fused_adam_cuda_kernel.cu:77-80,100-101,113-114,120-121,128-129
+    want = {"FULL_PRECISION": 4 * 4 + 3 * 4, "MIXED_PRECISION": (4 + 4 + 4 + 2) + (4 + 4 + 4 + 2),
+            "MEMORY_EFFICIENT_MIXED_PRECISION": (2 + 4 + 4 + 2) + (2 + 4 + 4), "PURE_FP16": 4 * 2 + 3 * 2}
+    assert bench.BYTES_PER_PARAM == want
+    assert bench.HBM_PEAK_GBS == 8000.0
