@@ -17,7 +17,7 @@ MEMORY_EFFICIENT_MIXED_PRECISION = 2
 PURE_FP16 = 3
 FULL_PRECISION_FP16_COPY = 4
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
 
@@ -83,6 +83,7 @@ SIGNATURES = {
     "fsadam_head_elems": (_i32, [ctypes.POINTER(FsAdamTensor), _i32, ctypes.POINTER(_i64)]),
     "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),
     "fsadam_grad_pass": (_i32, [ctypes.POINTER(FsGradTensor), _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _vp]),
+    "fsadam_grad_pass_noalloc": (_i32, [ctypes.POINTER(FsGradTensor), _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _vp]),
     "fsadam_clear_cache": (_i32, []),
     "fsadam_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
 }

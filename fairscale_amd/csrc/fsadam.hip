@@ -51,6 +51,20 @@
 #include "adam_kernels.h"
 #include "grad_kernels.h"
 
+// --------------------------------------------------------------------------------------------
+// fsadam_grad_pass_noalloc: device memory the library never allocates
+// --------------------------------------------------------------------------------------------
+// The descriptor table and the partial results of a gradient pass for callers that cannot allocate: one
+// array per GPU, part of the loaded code object, held until the process ends.  Layout: the table
+// (FSADAM_NOALLOC_MAX_DESCRIPTORS rows of 64 bytes), then the partials of the tiles' workgroups
+// (FSADAM_NOALLOC_MAX_WORKGROUPS), of the second reduction stage (512) and the total (1), 16 bytes each.
+// In host code the name below is only a handle for hipGetSymbolAddress: the device address is looked up
+// once per device (scratch_on_current_device) and only that pointer is ever handed to a kernel.
+constexpr size_t kScratchTableBytes = (size_t)FSADAM_NOALLOC_MAX_DESCRIPTORS * 64;
+constexpr size_t kScratchPartials = (size_t)FSADAM_NOALLOC_MAX_WORKGROUPS + 512 + 1;
+constexpr size_t kScratchBytes = kScratchTableBytes + kScratchPartials * 16;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 namespace {
 
 // --------------------------------------------------------------------------------------------
@@ -669,6 +683,37 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
     return L;
 }
 
+// The descriptors of a gradient list under layout L, written to table[0 .. L.descs()): large tensors first,
+// then the middle-sized ones, then one per tile.  False when the count does not come out as L says.
+bool grad_fill_table(ChunkDesc* table, const Layout& L, const FsGradTensor* grads, int64_t n, int esz, int64_t align_heads,
+                     int64_t unaligned_vectors) {
+    ChunkDesc* large = table;
+    ChunkDesc* mid = large + L.n_large_descs;
+    ChunkDesc* small = mid + L.n_mid_descs;
+    for (int64_t t = 0; t < n; ++t) {
+        const FsGradTensor& r = grads[t];
+        if (r.numel == 0) continue;
+        const int64_t head = grad_head_elems(r, esz, align_heads);
+        // pieces: the head (tile-sized descriptors), then the rest in shared chunks or tiles
+        const struct { int64_t start, count; int cls; } pieces[2] = {{0, head, kClassSmall}, {head, r.numel - head, class_of(r.numel - head, L)}};
+        for (const auto& piece : pieces) {
+            const int64_t chunk_elems = piece.cls == kClassLarge ? L.large_chunk_elems : piece.cls == kClassMid ? L.mid_chunk_elems : L.tile_elems;
+            const int64_t chunks = ceil_div(piece.count, chunk_elems);
+            ChunkDesc*& out = piece.cls == kClassLarge ? large : piece.cls == kClassMid ? mid : small;
+            for (int64_t c = 0; c < chunks; ++c) {
+                ChunkDesc& d = out[c];
+                std::memset(&d, 0, sizeof(d));
+                const int64_t first = piece.start + c * chunk_elems;
+                d.g = advance(r.g, first, esz);
+                d.n = (uint32_t)std::min<int64_t>(chunk_elems, piece.start + piece.count - first);
+                d.vector_ok = (unaligned_vectors != 0 || aligned_to(advance(r.g, piece.start, esz), 16)) ? 1u : 0u;
+            }
+            out += chunks;
+        }
+    }
+    return large == table + L.n_large_descs && mid == table + L.n_large_descs + L.n_mid_descs && small == table + L.descs();
+}
+
 void grad_plan_free(GradPlan* plan) {
     mark_destroy(plan->partials_mark);
     for (TableSlot& slot : plan->slots) slot_destroy(slot);
@@ -734,32 +779,7 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
         }
         plan->cap_partials = cap;
     }
-    const int esz = grad_elem_size(plan->dtype);
-    ChunkDesc* large = slot.h_table;
-    ChunkDesc* mid = large + L.n_large_descs;
-    ChunkDesc* small = mid + L.n_mid_descs;
-    for (int64_t t = 0; t < n; ++t) {
-        const FsGradTensor& r = grads[t];
-        if (r.numel == 0) continue;
-        const int64_t head = grad_head_elems(r, esz, plan->align_heads);
-        // pieces: the head (tile-sized descriptors), then the rest in shared chunks or tiles
-        const struct { int64_t start, count; int cls; } pieces[2] = {{0, head, kClassSmall}, {head, r.numel - head, class_of(r.numel - head, L)}};
-        for (const auto& piece : pieces) {
-            const int64_t chunk_elems = piece.cls == kClassLarge ? L.large_chunk_elems : piece.cls == kClassMid ? L.mid_chunk_elems : L.tile_elems;
-            const int64_t chunks = ceil_div(piece.count, chunk_elems);
-            ChunkDesc*& out = piece.cls == kClassLarge ? large : piece.cls == kClassMid ? mid : small;
-            for (int64_t c = 0; c < chunks; ++c) {
-                ChunkDesc& d = out[c];
-                std::memset(&d, 0, sizeof(d));
-                const int64_t first = piece.start + c * chunk_elems;
-                d.g = advance(r.g, first, esz);
-                d.n = (uint32_t)std::min<int64_t>(chunk_elems, piece.start + piece.count - first);
-                d.vector_ok = (plan->unaligned_vectors != 0 || aligned_to(advance(r.g, piece.start, esz), 16)) ? 1u : 0u;
-            }
-            out += chunks;
-        }
-    }
-    if (large != slot.h_table + L.n_large_descs || mid != slot.h_table + L.n_large_descs + L.n_mid_descs || small != slot.h_table + n_descs)
+    if (!grad_fill_table(slot.h_table, L, grads, n, grad_elem_size(plan->dtype), plan->align_heads, plan->unaligned_vectors))
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(grads, grads + n);
@@ -775,33 +795,25 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     return FSADAM_OK;
 }
 
+// The launches of one pass: the tiles (workgroups of `waves` consecutive tiles, one partial each, into
+// first[0 .. n_groups)), then two fixed-shape reduction steps through second[0 .. kReduceBlocks) and total[0],
+// the last of which publishes.  Shared by fsadam_grad_pass and its variant that allocates nothing.
 template <typename T>
-int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, int write_back, float* found_inf, double* sum_squares,
-                  float* abs_max, hipStream_t stream) {
-    const Layout& L = plan->layout;
+int grad_launch(const ChunkDesc* table, const Layout& L, int64_t waves, int64_t items, size_t lds, float inv_scale, const float* inv_scale_dev,
+                int write_back, GradPartial* first, GradPartial* second, GradPartial* total, float* found_inf, double* sum_squares,
+                float* abs_max, hipStream_t stream) {
     const int64_t n_blocks = L.blocks();
     const TileMap map = tile_map(L);
-    TableSlot& slot = plan->slots[plan->current];
-    GradPartial* first = plan->d_partials;
-    GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
-    GradPartial* total = second + kReduceBlocks;
-    int rc = mark_order_after(slot.mark, stream);
-    if (rc) return rc;
-    rc = mark_order_after(plan->partials_mark, stream);
-    if (rc) return rc;
-    // workgroups of `waves` consecutive tiles, one partial each
-    const int64_t waves = plan->waves;
     const int64_t n_groups = ceil_div(n_blocks, waves);
 #define FS_GRAD_LAUNCH(WAVES, ITEMS)                                                                                          \
     hipLaunchKernelGGL((fsadam_grad_tiles<T, WAVES, ITEMS>), dim3((uint32_t)n_groups), dim3(64 * WAVES), lds, stream,        \
-                       slot.d_table, map, (uint32_t)n_blocks, inv_scale, inv_scale_dev, write_back, first)
+                       table, map, (uint32_t)n_blocks, inv_scale, inv_scale_dev, write_back, first)
 #define FS_GRAD_ITEMS(WAVES)                          \
     do {                                              \
-        if (plan->items == 2) FS_GRAD_LAUNCH(WAVES, 2);      \
-        else if (plan->items == 8) FS_GRAD_LAUNCH(WAVES, 8); \
-        else FS_GRAD_LAUNCH(WAVES, 4);                       \
+        if (items == 2) FS_GRAD_LAUNCH(WAVES, 2);      \
+        else if (items == 8) FS_GRAD_LAUNCH(WAVES, 8); \
+        else FS_GRAD_LAUNCH(WAVES, 4);                 \
     } while (0)
-    const size_t lds = (size_t)plan->lds_throttle;
     if (n_blocks > 0) {
         if (waves == 16) FS_GRAD_ITEMS(16);
         else if (waves == 4) FS_GRAD_ITEMS(4);
@@ -818,9 +830,63 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total, 1, (int)(sizeof(T) == 2),
                        found_inf, sum_squares, abs_max);
     FS_HIP(hipGetLastError());
+    return FSADAM_OK;
+}
+
+template <typename T>
+int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, int write_back, float* found_inf, double* sum_squares,
+                  float* abs_max, hipStream_t stream) {
+    TableSlot& slot = plan->slots[plan->current];
+    GradPartial* first = plan->d_partials;
+    GradPartial* second = plan->d_partials + plan->cap_partials - kReduceBlocks - 1;
+    GradPartial* total = second + kReduceBlocks;
+    int rc = mark_order_after(slot.mark, stream);
+    if (rc) return rc;
+    rc = mark_order_after(plan->partials_mark, stream);
+    if (rc) return rc;
+    rc = grad_launch<T>(slot.d_table, plan->layout, plan->waves, plan->items, (size_t)plan->lds_throttle, inv_scale, inv_scale_dev, write_back,
+                        first, second, total, found_inf, sum_squares, abs_max, stream);
+    if (rc) return rc;
     rc = mark_use(slot.mark, stream, plan->lazy_events);
     if (rc) return rc;
     return mark_use(plan->partials_mark, stream, plan->lazy_events);
+}
+
+int validate_grads(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype) {
+    if (grad_dtype != FSADAM_GRAD_F32 && grad_dtype != FSADAM_GRAD_F16) return fail(FSADAM_EINVAL, "unknown gradient dtype " + std::to_string(grad_dtype));
+    if (n_tensors < 1) return fail(FSADAM_EINVAL, "gradient list is empty");
+    if (!grads) return fail(FSADAM_EINVAL, "grads is NULL");
+    for (int64_t t = 0; t < n_tensors; ++t) {
+        if (grads[t].numel < 0) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": negative numel");
+        if (grads[t].numel == 0) continue;
+        if (!grads[t].g) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": NULL pointer");
+        if (!aligned_to(grads[t].g, grad_elem_size(grad_dtype))) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": pointer not aligned to its element size");
+    }
+    return FSADAM_OK;
+}
+
+// ---- the variant of the gradient pass that allocates nothing ---------------------------------------
+
+static_assert(sizeof(GradPartial) == 16 && sizeof(ChunkDesc) == 64 && kReduceBlocks == 512, "the scratch array is sized for these");
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;                  // guards the two arrays below; held for the whole of a call
+unsigned char* g_scratch_ptr[kMaxDevices];   // device address of `scratch` on each GPU, once looked up
+ChunkDesc g_scratch_staging[FSADAM_NOALLOC_MAX_DESCRIPTORS];  // host side of the table, rebuilt by every call
+
+// Device address of this GPU's copy of `scratch` (every GPU that loads the library holds its own copy at
+// its own address).  The symbol is resolved once per device, with that device current.
+int scratch_on_current_device(unsigned char** out) {
+    int dev = -1;
+    FS_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(FSADAM_EINVAL, "device index " + std::to_string(dev) + " is beyond what this entry point keeps a scratch pointer for");
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        FS_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(FSADAM_EHIP, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return FSADAM_OK;
 }
 
 std::vector<GradPlan*> g_grad_cache;
@@ -1098,15 +1164,7 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
 
 int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
                      int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream) {
-    if (grad_dtype != FSADAM_GRAD_F32 && grad_dtype != FSADAM_GRAD_F16) return fail(FSADAM_EINVAL, "unknown gradient dtype " + std::to_string(grad_dtype));
-    if (n_tensors < 1) return fail(FSADAM_EINVAL, "gradient list is empty");
-    if (!grads) return fail(FSADAM_EINVAL, "grads is NULL");
-    for (int64_t t = 0; t < n_tensors; ++t) {
-        if (grads[t].numel < 0) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": negative numel");
-        if (grads[t].numel == 0) continue;
-        if (!grads[t].g) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": NULL pointer");
-        if (!aligned_to(grads[t].g, grad_elem_size(grad_dtype))) return fail(FSADAM_EINVAL, "gradient " + std::to_string(t) + ": pointer not aligned to its element size");
-    }
+    if (int bad = validate_grads(grads, n_tensors, grad_dtype)) return bad;
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
@@ -1158,6 +1216,49 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     return grad_dtype == FSADAM_GRAD_F16
                ? grad_plan_run<_Float16>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream)
                : grad_plan_run<float>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream);
+}
+
+int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
+                             int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream) {
+    if (int bad = validate_grads(grads, n_tensors, grad_dtype)) return bad;
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    // Shape: 16 tiles per workgroup whatever the kind of pass (one partial per workgroup keeps the scratch small);
+    // vectors per lane and ballast as fsadam_grad_pass chooses them.  Options are not consulted.
+    const bool writes = write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f);
+    const int64_t waves = 16, items = writes ? 4 : 8;
+    const size_t lds = writes ? 13312 : 16384;
+    const Layout L = grad_layout(grads, n_tensors, grad_dtype, items, kMaxLargeChunk, /*align_heads=*/1, /*mid_tiles=*/16);
+    const int64_t n_descs = L.descs(), n_groups = ceil_div(L.blocks(), waves);
+    if (n_descs > FSADAM_NOALLOC_MAX_DESCRIPTORS)
+        return fail(FSADAM_EINVAL, "gradient list needs " + std::to_string(n_descs) + " descriptors, fsadam_grad_pass_noalloc holds at most " +
+                                       std::to_string(FSADAM_NOALLOC_MAX_DESCRIPTORS) + " (use fsadam_grad_pass)");
+    if (n_groups > FSADAM_NOALLOC_MAX_WORKGROUPS)
+        return fail(FSADAM_EINVAL, "gradient list needs " + std::to_string(n_groups) + " workgroups, fsadam_grad_pass_noalloc holds partial results for at most " +
+                                       std::to_string(FSADAM_NOALLOC_MAX_WORKGROUPS) + " (use fsadam_grad_pass)");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    unsigned char* base = nullptr;
+    if (int rc = scratch_on_current_device(&base)) return rc;
+    ChunkDesc* table = reinterpret_cast<ChunkDesc*>(base);
+    GradPartial* first = reinterpret_cast<GradPartial*>(base + kScratchTableBytes);
+    GradPartial* second = first + FSADAM_NOALLOC_MAX_WORKGROUPS;
+    GradPartial* total = second + kReduceBlocks;
+    if (!grad_fill_table(g_scratch_staging, L, grads, n_tensors, grad_elem_size(grad_dtype), 1, 1))
+        return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
+    // The table travels in kernel arguments, kDescsPerPut rows per launch: no copy engine, no staging buffer of
+    // the runtime's, nothing a capture could not record.
+    for (int64_t at = 0; at < n_descs; at += kDescsPerPut) {
+        const int64_t count = std::min<int64_t>(kDescsPerPut, n_descs - at);
+        DescBatch batch;
+        std::memcpy(batch.rows, g_scratch_staging + at, (size_t)count * sizeof(ChunkDesc));
+        hipLaunchKernelGGL(fsadam_put_descs, dim3(1), dim3(64), 0, stream, table, batch, (uint32_t)at, (uint32_t)count);
+    }
+    FS_HIP(hipGetLastError());
+    // Every partial a reduction reads was written by this call's tiles; nothing in the scratch has to start at zero.
+    return grad_dtype == FSADAM_GRAD_F16
+               ? grad_launch<_Float16>(table, L, waves, items, lds, inv_scale, inv_scale_dev, write_back, first, second, total, found_inf_dev,
+                                       sum_squares_dev, abs_max_dev, stream)
+               : grad_launch<float>(table, L, waves, items, lds, inv_scale, inv_scale_dev, write_back, first, second, total, found_inf_dev,
+                                    sum_squares_dev, abs_max_dev, stream);
 }
 
 int fsadam_clear_cache(void) {

@@ -274,6 +274,19 @@ __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __r
     if (abs_max) *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)s_stored[0]) : __builtin_bit_cast(float, s_stored[0]);
 }
 
+// Rows of a descriptor table handed over in the kernel arguments and written to table[first .. first + count):
+// how a table reaches the device without a copy (3 KiB of arguments per launch).
+constexpr int kDescsPerPut = 48;
+struct DescBatch {
+    ChunkDesc rows[kDescsPerPut];
+};
+__global__ __launch_bounds__(64) void fsadam_put_descs(ChunkDesc* __restrict__ table, DescBatch batch, uint32_t first, uint32_t count) {
+    constexpr uint32_t kWords = sizeof(ChunkDesc) / sizeof(uint32_t);
+    gptr<uint32_t> out = (gptr<uint32_t>)reinterpret_cast<uint32_t*>(table + first);
+    const uint32_t* in = reinterpret_cast<const uint32_t*>(batch.rows);
+    for (uint32_t w = threadIdx.x; w < count * kWords; w += 64) out[w] = in[w];
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 template <int BLOCK>

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FSADAM_ABI_VERSION 2
+#define FSADAM_ABI_VERSION 3
 
 /* Precision modes = the four dtype combinations the reference dispatches on
  * (fairscale/clib/fused_adam_cuda/fused_adam_cuda_kernel.cu:172-256; Python enum
@@ -240,6 +240,26 @@ typedef struct FsGradTensor {
 
 int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
                      int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream);
+
+/* fsadam_grad_pass for callers that cannot allocate device memory: code that runs between the begin and end of
+ * a HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference
+ * (its gradient passes are torch operators, which allocate their outputs).  Same arguments, same results:
+ * what is stored, the flag and the maximum have the bits fsadam_grad_pass gives; the sum of squares is
+ * bit-identical for a pass that writes nothing back and within 1e-6 relative otherwise (16 tiles always share one
+ * partial here).  The call makes no hipMalloc / hipFree / hipHostMalloc, creates no stream or event and copies
+ * nothing with the copy engines: the descriptor table travels in kernel arguments (one small launch per 48
+ * rows) and lives, with the partial results, in an array that is part of the library's code object,
+ * FSADAM_NOALLOC_MAX_DESCRIPTORS * 64 + (FSADAM_NOALLOC_MAX_WORKGROUPS + 513) * 16 bytes (1.26 MiB) per GPU,
+ * held until the process ends.  A list that needs more descriptors or workgroups than that is refused with
+ * FSADAM_EINVAL (a workgroup covers 65536 fp16 / 32768 fp32 elements when the pass only reads, half as many
+ * when it writes back: at least 1.07e9 elements in every case; a tensor of 131072 elements or more takes one
+ * descriptor per 2^16..2^24 elements, smaller ones up to 16, plus one for a misaligned start).  Tuning options
+ * are not consulted.  All calls on one GPU share that GPU's array: calls whose kernels may overlap (different
+ * streams without an order between them, or two threads) race; calls on one stream are ordered by it. */
+#define FSADAM_NOALLOC_MAX_DESCRIPTORS 4096
+#define FSADAM_NOALLOC_MAX_WORKGROUPS 65536
+int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,
+                             int write_back, float* found_inf_dev, double* sum_squares_dev, float* abs_max_dev, void* hip_stream);
 
 /* Drops the tables cached by fsadam_step and fsadam_grad_pass (synchronises the devices that own them). */
 int fsadam_clear_cache(void);

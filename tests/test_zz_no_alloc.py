@@ -1,0 +1,126 @@
+"""``fsadam_grad_pass_noalloc`` (the gradient pass for callers that cannot allocate device memory) against
+``fsadam_grad_pass``, both through the C ABI.
+
+Bars: the gradients as stored, the overflow flag and the maximum are bit-identical; the sum of squares is
+bit-identical for a pass that only reads (same workgroup shape in both entry points) and within 1e-6
+relative for one that writes back (the variant always adds 16 tiles per partial).  Every case runs twice in
+a row through the variant, the second time on a smaller list, because the calls share one array per GPU that
+keeps the first call's table and partial results."""
+from __future__ import annotations
+
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _rows(tensors):
+    from fairscale_amd import _cabi
+
+    rows = (_cabi.FsGradTensor * len(tensors))()
+    for r, t in zip(rows, tensors):
+        r.g, r.numel = t.data_ptr(), t.numel()
+    return rows
+
+
+def _call(entry, tensors, inv_scale, write_back, inv_on_device=False):
+    from fairscale_amd import _cabi
+
+    L = _cabi.lib()
+    dev = tensors[0].device
+    flag = torch.zeros(1, dtype=torch.float32, device=dev)
+    ssq = torch.full((1,), -1.0, dtype=torch.float64, device=dev)
+    amax = torch.full((1,), -1.0, dtype=torch.float32, device=dev)
+    inv_dev = torch.tensor([inv_scale], dtype=torch.float32, device=dev) if inv_on_device else None
+    code = _cabi.GRAD_F16 if tensors[0].dtype == torch.float16 else _cabi.GRAD_F32
+    _cabi.check(getattr(L, entry)(_rows(tensors), len(tensors), code, 1.0 if inv_on_device else inv_scale,
+                                  inv_dev.data_ptr() if inv_on_device else None, 1 if write_back else 0, flag.data_ptr(),
+                                  ssq.data_ptr(), amax.data_ptr(), int(torch.cuda.current_stream(dev).cuda_stream)))
+    torch.cuda.synchronize()
+    return flag.item(), ssq.item(), amax.item()
+
+
+def _make(sizes, dtype, seed, device, offset=0, plant=None):
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    out = []
+    for n in sizes:
+        host = torch.randn(n + offset, generator=gen) * 0.05
+        if plant is not None and n > 3:
+            host[offset + n // 2] = plant
+        out.append(host.to(dtype).to(device)[offset:])
+    return out
+
+
+def _bits(t):
+    return t.cpu().numpy().view(np.uint16 if t.dtype == torch.float16 else np.uint32)
+
+
+def _compare(sizes, dtype, inv_scale, write_back, device, seed, offset=0, plant=None, inv_on_device=False):
+    a = _make(sizes, dtype, seed, device, offset, plant)
+    # A pass that writes nothing runs on the same memory in both entry points, and then every output must have the
+    # same bits (same tiles, same order of additions).  One that writes back needs a copy of its own.
+    writes = write_back and (inv_on_device or inv_scale != 1.0)
+    b = a if not writes else [torch.cat([torch.zeros(offset, dtype=dtype, device=device), t])[offset:] for t in a]
+    want = _call("fsadam_grad_pass", a, inv_scale, write_back, inv_on_device)
+    got = _call("fsadam_grad_pass_noalloc", b, inv_scale, write_back, inv_on_device)
+    what = f"sizes={sizes[:4]}.. dtype={dtype} inv={inv_scale} write_back={write_back} offset={offset}"
+    for x, y in zip(a, b):
+        assert np.array_equal(_bits(x), _bits(y)), what
+    assert got[0] == want[0], what
+    if np.isnan(want[2]):
+        assert np.isnan(got[2]) and np.isnan(got[1]), what
+    else:
+        assert got[2] == want[2], what
+        if writes:
+            assert abs(got[1] - want[1]) <= 1e-6 * abs(want[1]) or got[1] == want[1], what
+        else:
+            assert got[1] == want[1], what
+
+
+BIG = [3_000_001, 131072, 70001, 4096, 4097, 1, 0, 9, 2049, 650_000]
+SMALL = [70001, 5, 2048]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("write_back", [False, True])
+def test_two_calls_in_a_row_the_second_smaller(cuda_device, dtype, write_back):
+    for inv in (1.0, 1.0 / 64, 0.3):
+        print(f"[noalloc] dtype={dtype} write_back={write_back} inv={inv}", flush=True)
+        _compare(BIG, dtype, inv, write_back, cuda_device, seed=1)
+        _compare(SMALL, dtype, inv, write_back, cuda_device, seed=2)
+
+
+def test_views_between_cache_lines_and_a_scale_on_the_device(cuda_device):
+    print("[noalloc] misaligned views", flush=True)
+    _compare([300_001, 9000, 17], torch.float16, 0.25, True, cuda_device, seed=3, offset=3, inv_on_device=True)
+    _compare([9000], torch.float32, 0.3, False, cuda_device, seed=4, offset=1, inv_on_device=True)
+
+
+def test_non_finite_gradients_raise_the_flag(cuda_device):
+    print("[noalloc] non-finite", flush=True)
+    _compare([200_000, 77], torch.float16, 0.5, True, cuda_device, seed=5, plant=float("inf"))
+    _compare([5000], torch.float32, 1.0, False, cuda_device, seed=6, plant=float("nan"))
+
+
+def test_a_shard_sized_buffer_then_a_small_one(cuda_device):
+    print("[noalloc] shard", flush=True)
+    _compare([400_000_000], torch.float16, 1.0 / 1024, False, cuda_device, seed=7)
+    _compare([1000], torch.float16, 1.0 / 1024, False, cuda_device, seed=8)
+
+
+def test_lists_beyond_the_scratch_are_refused(cuda_device):
+    from fairscale_amd import _cabi
+
+    L = _cabi.lib()
+    # more descriptors than the array holds: 5000 small tensors (one descriptor each), no kernel is launched
+    many = [torch.zeros(8, dtype=torch.float16, device=cuda_device) for _ in range(5000)]
+    rc = L.fsadam_grad_pass_noalloc(_rows(many), len(many), _cabi.GRAD_F16, 1.0, None, 0, None, None, None, None)
+    assert rc == -1 and b"descriptors" in L.fsadam_last_error()
+    # more workgroups than there are partials: sizes only, the pointer is never followed
+    rows = (_cabi.FsGradTensor * 1)()
+    rows[0].g, rows[0].numel = many[0].data_ptr(), 3 * 10 ** 9
+    rc = L.fsadam_grad_pass_noalloc(rows, 1, _cabi.GRAD_F32, 0.5, None, 1, None, None, None, None)
+    assert rc == -1 and b"workgroups" in L.fsadam_last_error()
+    torch.cuda.synchronize()
