@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--calib-copy-bytes", type=int, default=0,
                     help="first run the library's plain copy kernel over this many bytes three times (a dispatch of known "
                          "traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (block, groups, lds_throttle, xcd_remap)")
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (lds_throttle, merge_runs, align_heads, mid_tiles, ...)")
     return ap.parse_args()
 
 
@@ -304,7 +304,7 @@ def main():
                    "storage": {"FULL_PRECISION": "p,g,m,v fp32", "MIXED_PRECISION": "p,m,v fp32; g, copy-out fp16",
                                "MEMORY_EFFICIENT_MIXED_PRECISION": "p,g fp16; m,v fp32", "PURE_FP16": "p,g,m,v fp16"}[args.mode], "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
                    "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
-                   "options": {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap")}},
+                   "options": {k: _cabi.get_option(k) for k in ("lds_throttle", "merge_runs", "align_heads", "mid_tiles")}},
         "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": load_traffic(workload),
                      "kernel": "fsadam_tiles", "kernel_ms": main_res["kernel_ms"], "bytes_per_param": main_res["bytes_per_param"]},

@@ -50,7 +50,7 @@ class FsAdamPlanInfo(_Int64Fields):
     _fields_ = [("mode", ctypes.c_int32), ("device", ctypes.c_int32)] + [
         (name, ctypes.c_int64)
         for name in ("n_tensors", "total_elems", "tile_elems", "large_chunk_elems", "n_descriptors", "n_vector_tensors",
-                     "n_scalar_tensors", "n_launches", "grid", "block", "lds_throttle", "uploads")
+                     "n_scalar_tensors", "n_launches", "grid", "block", "lds_throttle", "uploads", "n_runs")
     ]
 
 
@@ -59,7 +59,7 @@ class FsAdamLayout(_Int64Fields):
         (name, ctypes.c_int64)
         for name in ("tile_elems", "large_chunk_elems", "n_large_tensors", "n_small_tensors", "n_empty_tensors",
                      "n_large_descriptors", "n_small_descriptors", "grid_large", "grid_small", "mid_chunk_elems", "n_mid_tensors",
-                     "n_mid_descriptors", "grid_mid")
+                     "n_mid_descriptors", "grid_mid", "n_runs")
     ]
 
 
@@ -79,6 +79,7 @@ SIGNATURES = {
     # lr, beta1, beta2, eps, grad_scale_dev, optim_scale, decay, step, eps_mode, bias_correction, found_inf, stream
     "fsadam_plan_step_dev_scale": (_i32, [_vp, _f32, _f32, _f32, _f32, _vp, _f32, _f32, _i32, _i32, _i32, _vp, _vp]),
     "fsadam_plan_info": (_i32, [_vp, ctypes.POINTER(FsAdamPlanInfo)]),
+    "fsadam_plan_lazy_events": (_i32, [_vp, _i32]),
     "fsadam_plan_destroy": (_i32, [_vp]),
     "fsadam_head_elems": (_i32, [ctypes.POINTER(FsAdamTensor), _i32, ctypes.POINTER(_i64)]),
     "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),
@@ -116,11 +117,6 @@ def lib() -> ctypes.CDLL:
         got = L.fsadam_version()
         if got != ABI_VERSION:
             raise ImportError(f"libfsadam.so has ABI version {got}, this package expects {ABI_VERSION}")
-        # The streams this package hands to the library are torch's, which live as long as the process, so
-        # the library may record its events only when something has to wait for them (3 us less per step).
-        # A caller that steps on a torch.cuda.ExternalStream it destroys later sets the option back to 0.
-        if L.fsadam_set_option(b"lazy_events", 1) != 0:
-            raise ImportError("libfsadam.so does not know the option lazy_events")
         _lib = L
     return _lib
 

@@ -87,19 +87,14 @@ int fail_hip(hipError_t e, const char* what) {
     } while (0)
 
 struct Options {
-    int64_t block = 64;         // threads per workgroup: 64, 128 or 256
-    int64_t groups = 1;         // vectors per lane per stream: 1 or 2
     int64_t lds_throttle = -1;  // bytes of untouched LDS per workgroup (0 = no cap, -1 = per-mode default)
-    int64_t xcd_remap = 0;      // 0: tiles in dispatch order; R > 0: each XCD takes runs of R consecutive tiles
     int64_t grad_items = 0;     // gradient pass: 16-byte vectors per lane (2, 4 or 8; 0 = by kind of pass)
     int64_t grad_lds_throttle = -1;  // gradient pass: LDS ballast per workgroup (-1 = by kind of pass)
-    int64_t max_large_chunk = kMaxLargeChunk;  // elements per shared descriptor, upper bound (a power of two)
-    int64_t unaligned_vectors = 1;  // 1: full tiles of misaligned streams use vector instructions too; 0: element-wise
     int64_t grad_waves = 0;         // gradient pass: tiles (waves) per workgroup, 1, 4 or 16; 0 = by kind of pass
     int64_t mid_tiles = 16;         // tiles that share a descriptor of a middle-sized tensor (a power of two up to 64; 0 = no such class)
     int64_t upload_stream = 1;      // 1: tables are copied to the device on a stream of the library's own
-    int64_t lazy_events = 0;        // 1: events behind steps are recorded only when needed (streams must outlive the plan)
     int64_t align_heads = 1;        // 1: a tensor whose streams start off a cache line gives up a short head so that the rest starts on one
+    int64_t merge_runs = 1;         // 1: consecutive tensors that continue each other in every stream are laid out as one
 };
 
 // Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
@@ -223,6 +218,7 @@ struct Layout {
     int64_t tile_elems = 0;
     int64_t large_chunk_elems = 0;
     int64_t mid_chunk_elems = 0;  // 0: no middle class
+    int64_t n_runs = 0;  // rows after merging (fsadam: build_runs); the three classes below count these
     int64_t n_large = 0, n_mid = 0, n_small = 0, n_empty = 0;
     int64_t n_large_descs = 0, n_mid_descs = 0, n_small_descs = 0;
     int64_t total_elems = 0;
@@ -261,17 +257,44 @@ TileMap tile_map(const Layout& L) {
     return map;
 }
 
-Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Options& opt) {
-    Layout L;
-    L.tile_elems = opt.block * mode_elems(mode) * opt.groups;
-    L.mid_chunk_elems = mid_chunk_for(L.tile_elems, opt.mid_tiles);
-    int64_t min_large = 0;
+// Row b starts, in every stream, at the element behind row a's last one.
+bool continues(const FsAdamTensor& a, const FsAdamTensor& b, int mode) {
+    return advance(a.p, a.numel, size_p(mode)) == b.p && advance(a.m, a.numel, size_s(mode)) == b.m &&
+           advance(a.v, a.numel, size_s(mode)) == b.v && advance(a.g, a.numel, size_g(mode)) == b.g &&
+           (!mode_has_copy(mode) || advance(a.p_copy, a.numel, 2) == b.p_copy);
+}
+
+// The list as the layout sees it: empty rows dropped and, with option merge_runs, every maximal sequence of
+// consecutive rows that continue each other in all streams (parameters that are back-to-back views of one
+// buffer, with gradients and state laid out the same way, as OSS's buckets make them: oss.py:630-659,
+// param_bucket.py:62-90) replaced by ONE row over the whole sequence.  The update of an element does not
+// depend on where its tile starts, so the results are the same bits; what changes is that a list of
+// thousands of views becomes the few long runs a flat shard is.  run_of[t] (optional): index of the run
+// row t went into, -1 for an empty row.
+void build_runs(const FsAdamTensor* tensors, int64_t n, int mode, bool merge, std::vector<FsAdamTensor>& runs, std::vector<int64_t>* run_of) {
+    runs.clear();
+    if (run_of) run_of->assign((size_t)n, -1);
+    const FsAdamTensor* last = nullptr;  // the row the current run ends with
     for (int64_t t = 0; t < n; ++t) {
-        const int64_t numel = tensors[t].numel;
-        L.total_elems += numel;
-        if (numel == 0) { L.n_empty += 1; continue; }
-        const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
-        (row_vector_ok(tensors[t], mode, head) ? L.n_vector : L.n_scalar) += 1;
+        if (tensors[t].numel == 0) continue;
+        if (merge && last && continues(*last, tensors[t], mode)) runs.back().numel += tensors[t].numel;
+        else runs.push_back(tensors[t]);
+        last = &tensors[t];
+        if (run_of) (*run_of)[(size_t)t] = (int64_t)runs.size() - 1;
+    }
+}
+
+// `runs`: the rows build_runs made (none empty).
+Layout compute_layout(const std::vector<FsAdamTensor>& runs, int mode, const Options& opt) {
+    Layout L;
+    L.tile_elems = kBlock * mode_elems(mode);
+    L.mid_chunk_elems = mid_chunk_for(L.tile_elems, opt.mid_tiles);
+    L.n_runs = (int64_t)runs.size();
+    int64_t min_large = 0;
+    for (const FsAdamTensor& r : runs) {
+        L.total_elems += r.numel;
+        const int64_t head = head_elems(r, mode, opt), body = r.numel - head;
+        (row_vector_ok(r, mode, head) ? L.n_vector : L.n_scalar) += 1;
         const int cls = class_of(body, L);
         if (cls == kClassLarge) {
             L.n_large += 1;
@@ -281,11 +304,9 @@ Layout compute_layout(const FsAdamTensor* tensors, int64_t n, int mode, const Op
         }
     }
     // every large tensor spans at least two chunks, so the empty tiles after its end stay a small share
-    L.large_chunk_elems = std::min(opt.max_large_chunk, std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2)))));
-    for (int64_t t = 0; t < n; ++t) {
-        const int64_t numel = tensors[t].numel;
-        if (numel == 0) continue;
-        const int64_t head = head_elems(tensors[t], mode, opt), body = numel - head;
+    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
+    for (const FsAdamTensor& r : runs) {
+        const int64_t head = head_elems(r, mode, opt), body = r.numel - head;
         L.n_small_descs += ceil_div(head, L.tile_elems);
         const int cls = class_of(body, L);
         if (cls == kClassLarge) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
@@ -330,6 +351,8 @@ struct FsAdamPlan {
     Options opt;
     Layout layout;
     std::vector<FsAdamTensor> rows;  // what the current table was built from
+    std::vector<FsAdamTensor> runs;  // scratch of plan_set_tensors: the rows after merging
+    bool lazy_events = false;        // see UseMark; fsadam_plan_lazy_events
     int64_t uploads = 0;
     TableSlot slots[kTableSlots];
     int current = -1;  // slot holding the table of `rows`
@@ -444,7 +467,7 @@ void plan_release_buffers(FsAdamPlan* plan) {
 }
 
 // Descriptors for elements [start, start + count) of a tensor, chunk_elems each; returns how many.
-int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t start, int64_t count, int64_t chunk_elems, bool vec) {
+int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t start, int64_t count, int64_t chunk_elems) {
     const int64_t chunks = ceil_div(count, chunk_elems);
     for (int64_t c = 0; c < chunks; ++c) {
         const int64_t first = start + c * chunk_elems;
@@ -455,53 +478,41 @@ int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t star
         d.g = advance(r.g, first, size_g(mode));
         d.p_copy = mode_has_copy(mode) ? advance(r.p_copy, first, 2) : nullptr;
         d.n = (uint32_t)std::min<int64_t>(chunk_elems, start + count - first);
-        d.vector_ok = vec ? 1u : 0u;
+        d.pad32 = 0;
         d.pad = 0;
     }
     return chunks;
 }
 
-template <int MODE, int BLOCK, int GROUPS>
+template <int MODE>
 int launch_tiles(const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf, hipStream_t stream) {
     const int64_t n_blocks = L.blocks();
     if (n_blocks == 0) return FSADAM_OK;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
-    uint32_t grid = (uint32_t)n_blocks, xcd_stride = 0;
-    if (opt.xcd_remap) {  // value = tiles per run; 1 would be the identity
-        xcd_stride = (uint32_t)std::min<int64_t>(opt.xcd_remap, ceil_div(n_blocks, 8));
-        grid = (uint32_t)(ceil_div(n_blocks, 8 * (int64_t)xcd_stride) * 8 * xcd_stride);
-    }
-    hipLaunchKernelGGL((fsadam_tiles<MODE, BLOCK, GROUPS>), dim3(grid), dim3(BLOCK), (size_t)opt.lds_throttle, stream, table, tile_map(L),
-                       (uint32_t)n_blocks, xcd_stride, s, found_inf);
+    hipLaunchKernelGGL((fsadam_tiles<MODE, kBlock, 1>), dim3((uint32_t)n_blocks), dim3(kBlock), (size_t)opt.lds_throttle, stream, table, tile_map(L), s,
+                       found_inf);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
-}
-
-template <int MODE>
-int launch_shape(const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf, hipStream_t stream) {
-#define FS_CASE(B, G)                      \
-    if (opt.block == B && opt.groups == G) \
-    return launch_tiles<MODE, B, G>(table, L, opt, s, found_inf, stream)
-    FS_CASE(64, 1); FS_CASE(64, 2); FS_CASE(128, 1); FS_CASE(128, 2); FS_CASE(256, 1); FS_CASE(256, 2);
-#undef FS_CASE
-    return fail(FSADAM_EINVAL, "unsupported block/groups combination");
 }
 
 int launch_mode(int mode, const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf,
                 hipStream_t stream) {
 #define FS_MODE(M) \
-    case M: return launch_shape<M>(table, L, opt, s, found_inf, stream)
+    case M: return launch_tiles<M>(table, L, opt, s, found_inf, stream)
     switch (mode) {
         FS_MODE(FSADAM_FULL_PRECISION);
         FS_MODE(FSADAM_MIXED_PRECISION);
         FS_MODE(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION);
         FS_MODE(FSADAM_FULL_PRECISION_FP16_COPY);
-        default: return launch_shape<FSADAM_PURE_FP16>(table, L, opt, s, found_inf, stream);
+        default: return launch_tiles<FSADAM_PURE_FP16>(table, L, opt, s, found_inf, stream);
     }
 #undef FS_MODE
 }
 
+// On failure the plan is left without tensors (plan_step refuses) rather than with a layout that does not
+// belong to the table on the device.
 int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, hipStream_t stream) {
+    plan->rows.clear();
     int rc = validate_rows(tensors, n, plan->mode);
     if (rc) return rc;
     rc = refuse_capture(stream);
@@ -517,7 +528,9 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
         plan->opt = g_opt;
     }
     if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
-    const Layout L = compute_layout(tensors, n, plan->mode, plan->opt);
+    build_runs(tensors, n, plan->mode, plan->opt.merge_runs != 0, plan->runs, nullptr);
+    Layout L = compute_layout(plan->runs, plan->mode, plan->opt);
+    for (int64_t t = 0; t < n; ++t) L.n_empty += tensors[t].numel == 0 ? 1 : 0;
     const int64_t n_descs = L.descs();
     if (L.blocks() > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
@@ -545,30 +558,28 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     ChunkDesc* large = slot.h_table;
     ChunkDesc* mid = large + L.n_large_descs;
     ChunkDesc* small = mid + L.n_mid_descs;
-    for (int64_t t = 0; t < n; ++t) {
-        const FsAdamTensor& r = tensors[t];
-        if (r.numel == 0) continue;
+    for (const FsAdamTensor& r : plan->runs) {
         const int64_t head = head_elems(r, plan->mode, plan->opt), body = r.numel - head;
-        const bool vec = plan->opt.unaligned_vectors != 0 || row_vector_ok(r, plan->mode, head);
-        small += fill_descs(small, r, plan->mode, 0, head, L.tile_elems, plan->opt.unaligned_vectors != 0);
+        small += fill_descs(small, r, plan->mode, 0, head, L.tile_elems);
         const int cls = class_of(body, L);
-        if (cls == kClassLarge) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems, vec);
-        else if (cls == kClassMid) mid += fill_descs(mid, r, plan->mode, head, body, L.mid_chunk_elems, vec);
-        else small += fill_descs(small, r, plan->mode, head, body, L.tile_elems, vec);
+        if (cls == kClassLarge) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems);
+        else if (cls == kClassMid) mid += fill_descs(mid, r, plan->mode, head, body, L.mid_chunk_elems);
+        else small += fill_descs(small, r, plan->mode, head, body, L.tile_elems);
     }
     if (large != slot.h_table + L.n_large_descs || mid != slot.h_table + L.n_large_descs + L.n_mid_descs || small != slot.h_table + n_descs)
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
-    plan->layout = L;
-    plan->rows.assign(tensors, tensors + n);
     rc = upload_table(&plan->upload_stream, plan->opt.upload_stream != 0, slot, n_descs, stream);
     if (rc) return rc;
-    rc = mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
+    rc = mark_use(slot.mark, stream, plan->lazy_events);
     if (rc) return rc;
     // the steps that used the table this one replaces are all enqueued: their slot's event can be taken now
     if (plan->current >= 0) {
         rc = mark_settle(plan->slots[plan->current].mark);
         if (rc) return rc;
     }
+    // everything went through: the plan now describes the new table
+    plan->layout = L;
+    plan->rows.assign(tensors, tensors + n);
     plan->current = (plan->current + 1) % kTableSlots;
     plan->uploads += 1;
     return FSADAM_OK;
@@ -606,7 +617,7 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     if (rc) return rc;
     rc = launch_mode(plan->mode, slot.d_table, L, plan->opt, s, found_inf, stream);
     if (rc) return rc;
-    return mark_use(slot.mark, stream, plan->opt.lazy_events != 0);
+    return mark_use(slot.mark, stream, plan->lazy_events);
 }
 
 
@@ -617,11 +628,8 @@ struct GradPlan {
     int dtype = 0;
     int64_t items = 4;
     int64_t lds_throttle = 0;
-    int64_t max_large_chunk = kMaxLargeChunk;
-    int64_t unaligned_vectors = 1;
     int64_t align_heads = 1;
     int64_t mid_tiles = 16;
-    bool lazy_events = false;
     bool own_upload_stream = true;
     hipStream_t upload_stream = nullptr;
     int64_t waves = 1;  // tiles per workgroup: 1, 4 or 16
@@ -648,8 +656,7 @@ int64_t grad_head_elems(const FsGradTensor& r, int elem_size, int64_t align_head
     return (int64_t)(((1024 - (a & 1023u)) & 1023u) / (uintptr_t)elem_size);
 }
 
-Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t max_large_chunk, int64_t align_heads,
-                   int64_t mid_tiles) {
+Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t items, int64_t align_heads, int64_t mid_tiles) {
     Layout L;
     L.tile_elems = grad_tile_elems(dtype, items);
     L.mid_chunk_elems = mid_chunk_for(L.tile_elems, mid_tiles);
@@ -669,7 +676,7 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
             (cls == kClassMid ? L.n_mid : L.n_small) += 1;
         }
     }
-    L.large_chunk_elems = std::min(max_large_chunk, std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2)))));
+    L.large_chunk_elems = std::max(kMinLargeChunk, std::min(kMaxLargeChunk, floor_pow2(std::max<int64_t>(1, min_large / 2))));
     for (int64_t t = 0; t < n; ++t) {
         const int64_t numel = grads[t].numel;
         if (numel == 0) continue;
@@ -685,8 +692,7 @@ Layout grad_layout(const FsGradTensor* grads, int64_t n, int dtype, int64_t item
 
 // The descriptors of a gradient list under layout L, written to table[0 .. L.descs()): large tensors first,
 // then the middle-sized ones, then one per tile.  False when the count does not come out as L says.
-bool grad_fill_table(ChunkDesc* table, const Layout& L, const FsGradTensor* grads, int64_t n, int esz, int64_t align_heads,
-                     int64_t unaligned_vectors) {
+bool grad_fill_table(ChunkDesc* table, const Layout& L, const FsGradTensor* grads, int64_t n, int esz, int64_t align_heads) {
     ChunkDesc* large = table;
     ChunkDesc* mid = large + L.n_large_descs;
     ChunkDesc* small = mid + L.n_mid_descs;
@@ -706,7 +712,6 @@ bool grad_fill_table(ChunkDesc* table, const Layout& L, const FsGradTensor* grad
                 const int64_t first = piece.start + c * chunk_elems;
                 d.g = advance(r.g, first, esz);
                 d.n = (uint32_t)std::min<int64_t>(chunk_elems, piece.start + piece.count - first);
-                d.vector_ok = (unaligned_vectors != 0 || aligned_to(advance(r.g, piece.start, esz), 16)) ? 1u : 0u;
             }
             out += chunks;
         }
@@ -724,23 +729,19 @@ void grad_plan_free(GradPlan* plan) {
 
 // Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
 // a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
-void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* max_large_chunk, int64_t* unaligned_vectors, int64_t* waves,
-                int64_t* align_heads, int64_t* lazy_events, int64_t* mid_tiles, int64_t* upload_stream) {
+void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* waves, int64_t* align_heads, int64_t* mid_tiles, int64_t* upload_stream) {
     std::lock_guard<std::mutex> lock(g_mutex);
     *upload_stream = g_opt.upload_stream;
     *mid_tiles = g_opt.mid_tiles;
     *align_heads = g_opt.align_heads;
-    *lazy_events = g_opt.lazy_events;
     // a pass that only reads pays for every small store it makes: 16 tiles share one partial
     *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
-    *max_large_chunk = g_opt.max_large_chunk;
-    *unaligned_vectors = g_opt.unaligned_vectors;
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
     *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 13312 : 16384);
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
-    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->max_large_chunk, plan->align_heads, plan->mid_tiles);
+    const Layout L = grad_layout(grads, n, plan->dtype, plan->items, plan->align_heads, plan->mid_tiles);
     const int64_t n_blocks = L.blocks();
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "gradient list too large for one launch");
     const int64_t n_descs = L.descs();
@@ -779,13 +780,13 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
         }
         plan->cap_partials = cap;
     }
-    if (!grad_fill_table(slot.h_table, L, grads, n, grad_elem_size(plan->dtype), plan->align_heads, plan->unaligned_vectors))
+    if (!grad_fill_table(slot.h_table, L, grads, n, grad_elem_size(plan->dtype), plan->align_heads))
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     plan->layout = L;
     plan->rows.assign(grads, grads + n);
     rc = upload_table(&plan->upload_stream, plan->own_upload_stream, slot, n_descs, stream);
     if (rc) return rc;
-    rc = mark_use(slot.mark, stream, plan->lazy_events);
+    rc = mark_use(slot.mark, stream, false);
     if (rc) return rc;
     if (plan->current >= 0) {
         rc = mark_settle(plan->slots[plan->current].mark);
@@ -847,9 +848,9 @@ int grad_plan_run(GradPlan* plan, float inv_scale, const float* inv_scale_dev, i
     rc = grad_launch<T>(slot.d_table, plan->layout, plan->waves, plan->items, (size_t)plan->lds_throttle, inv_scale, inv_scale_dev, write_back,
                         first, second, total, found_inf, sum_squares, abs_max, stream);
     if (rc) return rc;
-    rc = mark_use(slot.mark, stream, plan->lazy_events);
+    rc = mark_use(slot.mark, stream, false);
     if (rc) return rc;
-    return mark_use(plan->partials_mark, stream, plan->lazy_events);
+    return mark_use(plan->partials_mark, stream, false);
 }
 
 int validate_grads(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype) {
@@ -914,9 +915,8 @@ bool same_rows(const FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n) {
 }
 
 bool same_options(const Options& a, const Options& b) {
-    return a.block == b.block && a.groups == b.groups && a.lds_throttle == b.lds_throttle && a.xcd_remap == b.xcd_remap &&
-           a.max_large_chunk == b.max_large_chunk && a.unaligned_vectors == b.unaligned_vectors && a.align_heads == b.align_heads &&
-           a.mid_tiles == b.mid_tiles;
+    return a.lds_throttle == b.lds_throttle && a.align_heads == b.align_heads && a.mid_tiles == b.mid_tiles && a.merge_runs == b.merge_runs &&
+           a.upload_stream == b.upload_stream;
 }
 
 }  // namespace
@@ -943,37 +943,21 @@ int fsadam_set_option(const char* name, int64_t value) {
     if (!name) return fail(FSADAM_EINVAL, "option name is NULL");
     std::lock_guard<std::mutex> lock(g_mutex);
     const std::string k(name);
-    if (k == "block") {
-        if (value != 64 && value != 128 && value != 256) return fail(FSADAM_EINVAL, "block must be 64, 128 or 256");
-        g_opt.block = value;
-    } else if (k == "groups") {
-        if (value != 1 && value != 2) return fail(FSADAM_EINVAL, "groups must be 1 or 2");
-        g_opt.groups = value;
-    } else if (k == "lds_throttle") {
+    if (k == "lds_throttle") {
         if (value < -1 || value > 65536) return fail(FSADAM_EINVAL, "lds_throttle must be -1 (per-mode default) or in [0, 65536] bytes");
         g_opt.lds_throttle = value;
-    } else if (k == "xcd_remap") {
-        if (value < 0 || value > (1 << 28)) return fail(FSADAM_EINVAL, "xcd_remap must be 0 (off) or a run length in tiles");
-        g_opt.xcd_remap = value;
-    } else if (k == "unaligned_vectors") {
-        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "unaligned_vectors must be 0 or 1");
-        g_opt.unaligned_vectors = value;
     } else if (k == "align_heads") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "align_heads must be 0 or 1");
         g_opt.align_heads = value;
+    } else if (k == "merge_runs") {
+        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "merge_runs must be 0 or 1");
+        g_opt.merge_runs = value;
     } else if (k == "mid_tiles") {
         if (value < 0 || value > 64 || (value & (value - 1)) != 0) return fail(FSADAM_EINVAL, "mid_tiles must be 0 or a power of two up to 64");
         g_opt.mid_tiles = value;
     } else if (k == "upload_stream") {
         if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "upload_stream must be 0 or 1");
         g_opt.upload_stream = value;
-    } else if (k == "lazy_events") {
-        if (value != 0 && value != 1) return fail(FSADAM_EINVAL, "lazy_events must be 0 or 1");
-        g_opt.lazy_events = value;
-    } else if (k == "max_large_chunk") {
-        if (value < 4096 || value > kMaxLargeChunk || (value & (value - 1)) != 0)
-            return fail(FSADAM_EINVAL, "max_large_chunk must be a power of two in [4096, 2^24] elements");
-        g_opt.max_large_chunk = value;
     } else if (k == "grad_items") {
         if (value != 0 && value != 2 && value != 4 && value != 8) return fail(FSADAM_EINVAL, "grad_items must be 0 (automatic), 2, 4 or 8");
         g_opt.grad_items = value;
@@ -993,14 +977,9 @@ int fsadam_get_option(const char* name, int64_t* value) {
     if (!name || !value) return fail(FSADAM_EINVAL, "NULL argument");
     std::lock_guard<std::mutex> lock(g_mutex);
     const std::string k(name);
-    if (k == "block") *value = g_opt.block;
-    else if (k == "groups") *value = g_opt.groups;
-    else if (k == "lds_throttle") *value = g_opt.lds_throttle;
-    else if (k == "xcd_remap") *value = g_opt.xcd_remap;
-    else if (k == "max_large_chunk") *value = g_opt.max_large_chunk;
-    else if (k == "unaligned_vectors") *value = g_opt.unaligned_vectors;
+    if (k == "lds_throttle") *value = g_opt.lds_throttle;
     else if (k == "align_heads") *value = g_opt.align_heads;
-    else if (k == "lazy_events") *value = g_opt.lazy_events;
+    else if (k == "merge_runs") *value = g_opt.merge_runs;
     else if (k == "upload_stream") *value = g_opt.upload_stream;
     else if (k == "mid_tiles") *value = g_opt.mid_tiles;
     else if (k == "grad_items") *value = g_opt.grad_items;
@@ -1020,12 +999,15 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
         std::lock_guard<std::mutex> lock(g_mutex);
         opt = g_opt;
     }
-    const Layout L = compute_layout(tensors, n_tensors, precision_mode, opt);
+    std::vector<FsAdamTensor> runs;
+    std::vector<int64_t> run_of;
+    build_runs(tensors, n_tensors, precision_mode, opt.merge_runs != 0, runs, &run_of);
+    const Layout L = compute_layout(runs, precision_mode, opt);
     out->tile_elems = L.tile_elems;
     out->large_chunk_elems = L.large_chunk_elems;
     out->n_large_tensors = L.n_large;
     out->n_small_tensors = L.n_small;
-    out->n_empty_tensors = L.n_empty;
+    out->n_empty_tensors = 0;
     out->n_large_descriptors = L.n_large_descs;
     out->n_small_descriptors = L.n_small_descs;
     out->grid_large = L.large_blocks();
@@ -1034,10 +1016,14 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
     out->n_mid_tensors = L.n_mid;
     out->n_mid_descriptors = L.n_mid_descs;
     out->grid_mid = L.mid_blocks();
+    out->n_runs = L.n_runs;
     for (int64_t t = 0; t < n_tensors; ++t) {
-        const int64_t head = tensors[t].numel > 0 ? head_elems(tensors[t], precision_mode, opt) : 0;
-        if (tensor_class) tensor_class[t] = tensors[t].numel == 0 ? 0 : (uint8_t)class_of(tensors[t].numel - head, L);
-        if (vector_ok) vector_ok[t] = (tensors[t].numel > 0 && row_vector_ok(tensors[t], precision_mode, head)) ? 1 : 0;
+        if (tensors[t].numel == 0) out->n_empty_tensors += 1;
+        // a tensor is laid out with the run it belongs to
+        const FsAdamTensor* run = run_of[(size_t)t] >= 0 ? &runs[(size_t)run_of[(size_t)t]] : nullptr;
+        const int64_t head = run ? head_elems(*run, precision_mode, opt) : 0;
+        if (tensor_class) tensor_class[t] = run ? (uint8_t)class_of(run->numel - head, L) : 0;
+        if (vector_ok) vector_ok[t] = (run && row_vector_ok(*run, precision_mode, head)) ? 1 : 0;
     }
     return FSADAM_OK;
 }
@@ -1062,6 +1048,17 @@ int fsadam_plan_create(int precision_mode, FsAdamPlan** out) {
     if (!plan) return fail(FSADAM_ENOMEM, "out of host memory");
     plan->mode = precision_mode;
     *out = plan;
+    return FSADAM_OK;
+}
+
+int fsadam_plan_lazy_events(FsAdamPlan* plan, int on) {
+    if (!plan) return fail(FSADAM_EINVAL, "plan is NULL");
+    if (on != 0 && on != 1) return fail(FSADAM_EINVAL, "lazy_events must be 0 or 1");
+    if (!on) {  // from now on every use is followed by its event: catch up on the ones that are owed
+        for (TableSlot& slot : plan->slots)
+            if (int rc = mark_settle(slot.mark)) return rc;
+    }
+    plan->lazy_events = on != 0;
     return FSADAM_OK;
 }
 
@@ -1103,7 +1100,8 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
     out->n_scalar_tensors = L.n_scalar;
     out->n_launches = L.descs() > 0 ? 1 : 0;
     out->grid = L.blocks();
-    out->block = plan->opt.block;
+    out->block = kBlock;
+    out->n_runs = L.n_runs;
     out->lds_throttle = plan->opt.lds_throttle;
     out->uploads = plan->uploads;
     return FSADAM_OK;
@@ -1169,15 +1167,14 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
     FS_HIP(hipGetDevice(&dev));
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     if (int refused = refuse_capture(stream)) return refused;  // its partial sums are guarded by events the host waits on
-    int64_t cur_items, cur_lds, cur_chunk, cur_unaligned, cur_waves, cur_heads, cur_lazy, cur_mid, cur_upload;
-    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_chunk, &cur_unaligned,
-               &cur_waves, &cur_heads, &cur_lazy, &cur_mid, &cur_upload);
+    int64_t cur_items, cur_lds, cur_waves, cur_heads, cur_mid, cur_upload;
+    grad_shape(write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f), &cur_items, &cur_lds, &cur_waves, &cur_heads, &cur_mid, &cur_upload);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     GradPlan* hit = nullptr;
     GradPlan* victim = nullptr;
     for (GradPlan* c : g_grad_cache) {
         if (c->device == dev && c->dtype == grad_dtype && c->items == cur_items && c->lds_throttle == cur_lds &&
-            c->max_large_chunk == cur_chunk && c->unaligned_vectors == cur_unaligned && c->waves == cur_waves && c->align_heads == cur_heads && c->mid_tiles == cur_mid && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
+            c->waves == cur_waves && c->align_heads == cur_heads && c->mid_tiles == cur_mid && same_grad_rows(c, grads, n_tensors)) { hit = c; break; }
         if (c->device == dev && c->dtype == grad_dtype && (!victim || c->lru < victim->lru)) victim = c;
     }
     if (!hit) {
@@ -1200,19 +1197,15 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
         }
         victim->items = cur_items;
         victim->lds_throttle = cur_lds;
-        victim->max_large_chunk = cur_chunk;
-        victim->unaligned_vectors = cur_unaligned;
         victim->align_heads = cur_heads;
         victim->mid_tiles = cur_mid;
         victim->own_upload_stream = cur_upload != 0;
-        victim->lazy_events = cur_lazy != 0;
         victim->waves = cur_waves;
         int rc = grad_plan_set(victim, grads, n_tensors, stream);
         if (rc) { victim->rows.clear(); return rc; }
         hit = victim;
     }
     hit->lru = ++g_tick;
-    hit->lazy_events = cur_lazy != 0;
     return grad_dtype == FSADAM_GRAD_F16
                ? grad_plan_run<_Float16>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream)
                : grad_plan_run<float>(hit, inv_scale, inv_scale_dev, write_back, found_inf_dev, sum_squares_dev, abs_max_dev, stream);
@@ -1227,7 +1220,7 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
     const bool writes = write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f);
     const int64_t waves = 16, items = writes ? 4 : 8;
     const size_t lds = writes ? 13312 : 16384;
-    const Layout L = grad_layout(grads, n_tensors, grad_dtype, items, kMaxLargeChunk, /*align_heads=*/1, /*mid_tiles=*/16);
+    const Layout L = grad_layout(grads, n_tensors, grad_dtype, items, /*align_heads=*/1, /*mid_tiles=*/16);
     const int64_t n_descs = L.descs(), n_groups = ceil_div(L.blocks(), waves);
     if (n_descs > FSADAM_NOALLOC_MAX_DESCRIPTORS)
         return fail(FSADAM_EINVAL, "gradient list needs " + std::to_string(n_descs) + " descriptors, fsadam_grad_pass_noalloc holds at most " +
@@ -1242,7 +1235,7 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
     GradPartial* first = reinterpret_cast<GradPartial*>(base + kScratchTableBytes);
     GradPartial* second = first + FSADAM_NOALLOC_MAX_WORKGROUPS;
     GradPartial* total = second + kReduceBlocks;
-    if (!grad_fill_table(g_scratch_staging, L, grads, n_tensors, grad_elem_size(grad_dtype), 1, 1))
+    if (!grad_fill_table(g_scratch_staging, L, grads, n_tensors, grad_elem_size(grad_dtype), 1))
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     // The table travels in kernel arguments, kDescsPerPut rows per launch: no copy engine, no staging buffer of
     // the runtime's, nothing a capture could not record.

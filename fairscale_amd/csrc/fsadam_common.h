@@ -15,7 +15,8 @@ namespace {
 
 constexpr int64_t kLargeThreshold = 131072;   // tensors with at least this many elements share descriptors
 constexpr int64_t kMinLargeChunk = 65536;     // elements per shared descriptor, lower bound
-constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room); option max_large_chunk lowers it
+constexpr int64_t kMaxLargeChunk = 1 << 24;   // upper bound (keeps the per-chunk count in 32 bits with room)
+constexpr int kBlock = 64;                    // threads per workgroup of the step: one wave64 (128 and 256 measured no faster)
 
 struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points at the chunk's first element
     void* p;
@@ -24,7 +25,7 @@ struct alignas(64) ChunkDesc {  // one per chunk; every pointer already points a
     const void* g;
     void* p_copy;
     uint32_t n;          // elements in this chunk (<= chunk size of its launch)
-    uint32_t vector_ok;  // full tiles of this chunk take the vector path
+    uint32_t pad32;
     uint64_t pad;
 };
 static_assert(sizeof(ChunkDesc) == 64, "descriptor must stay 64 bytes");

@@ -83,12 +83,13 @@ __device__ __forceinline__ uint32_t grad_word(uint32_t w, float inv_scale, f16x2
     return out;
 }
 
+// one half on its own (ragged tiles); the two scaled forms give the same bits.  Not grad_word on a word padded with a
+// zero: under an infinite factor the padding would turn into 0 * inf = NaN and spoil the sum.
 __device__ __forceinline__ _Float16 grad_scalar(_Float16 g, int how, float inv_scale, GradAcc& acc) {
-    const uint32_t w = __builtin_bit_cast(uint16_t, g);
-    uint32_t out;
-    if (how == kGradUnit) out = grad_word<kGradUnit>(w, inv_scale, f16x2{}, acc);
-    else out = grad_word<kGradFloatScale>(w, inv_scale, f16x2{}, acc);  // the two scaled forms give the same bits
-    return __builtin_bit_cast(_Float16, (uint16_t)out);
+    acc.incoming_max = max_u16x2(acc.incoming_max, (uint32_t)__builtin_bit_cast(uint16_t, g) & 0x7fffu);
+    const _Float16 r = how == kGradUnit ? g : (_Float16)as_float32((float)g * inv_scale);
+    acc.sum = __builtin_fmaf((float)r, (float)r, acc.sum);
+    return r;
 }
 
 template <int HOW>
@@ -113,7 +114,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint
     using u32x4_in_memory = typename GradTraits<T>::in_memory;
     const uint32_t left = d.n - off;
     gptr<T> g = (gptr<T>)const_cast<void*>(d.g) + off;
-    if (d.vector_ok && left >= kTile) {
+    if (left >= kTile) {
         u32x4 raw[ITEMS];
 #pragma unroll
         for (int k = 0; k < ITEMS; ++k)
@@ -133,8 +134,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint
                 __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + lane) * E));
         }
     } else {
-        const uint32_t count = left < kTile ? left : kTile;
-        for (uint32_t e = lane; e < count; e += BLOCK) {
+        for (uint32_t e = lane; e < left; e += BLOCK) {
             const T r = grad_scalar(g[e], HOW, inv_scale, acc);
             if (WRITE && HOW != kGradUnit) g[e] = r;
         }
@@ -271,7 +271,13 @@ __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __r
     const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
     if (s_incoming[0] >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
     if (sum_squares) *sum_squares = s_sum[0];
-    if (abs_max) *abs_max = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)s_stored[0]) : __builtin_bit_cast(float, s_stored[0]);
+    // The stored maximum was formed from the largest incoming magnitude, which is right whenever g -> dtype(g * inv_scale)
+    // is monotone in |g|.  An infinite or NaN inv_scale breaks that: a zero gradient then stores NaN (0 * inf) while the
+    // largest one stores inf.  Squares are never negative, so the sum is NaN exactly when some stored value is NaN:
+    // that is when the maximum is NaN too (torch's abs().max() propagates it).
+    float top = is_half ? (float)__builtin_bit_cast(_Float16, (uint16_t)s_stored[0]) : __builtin_bit_cast(float, s_stored[0]);
+    if (s_sum[0] != s_sum[0]) top = __builtin_nanf("");
+    if (abs_max) *abs_max = top;
 }
 
 // Rows of a descriptor table handed over in the kernel arguments and written to table[first .. first + count):

@@ -26,31 +26,46 @@ _lib.fsadam_last_error.restype = ctypes.c_char_p
 _F32, _F16 = torch.float32, torch.float16
 
 
+# element types of [p, m, v, g(, p_copy)] per FSADAM_* code: the combinations fused_adam_cuda_kernel.cu:165-263 dispatches on
+_DTYPES = {0: (_F32, _F32, _F32, _F32), 1: (_F32, _F32, _F32, _F16, _F16), 2: (_F16, _F32, _F32, _F16), 3: (_F16, _F16, _F16, _F16)}
+
+
 def _mode(lists):
-    """The dtype dispatch of fused_adam_cuda_kernel.cu:172-256, as FSADAM_* codes."""
-    p, m = lists[0][0].dtype, lists[1][0].dtype
-    if len(lists) == 5:
-        return 1  # FSADAM_MIXED_PRECISION
-    if p == _F32:
-        return 0  # FSADAM_FULL_PRECISION
-    return 2 if m == _F32 else 3  # FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION / FSADAM_PURE_FP16
+    """The dtype dispatch of fused_adam_cuda_kernel.cu:165-263 on the first tensor of each list, as FSADAM_* codes."""
+    if len(lists) not in (4, 5) or len(lists[0]) == 0:
+        raise RuntimeError("tensor_lists must be 4 or 5 non-empty lists")  # multi_tensor_apply.cuh:49-51
+    first = tuple(lst[0].dtype for lst in lists)
+    for code, dtypes in _DTYPES.items():
+        if first == dtypes:
+            return code
+    raise RuntimeError(f"no kernel for tensor lists of dtypes {first}")  # kernel.cu:167-176,196-199,258,261
 
 
 def adam(chunk_size, noop_flag, tensor_lists, lr, beta1, beta2, eps, grad_scale, optim_scale, found_inf, step, mode,
          bias_correction, decay):
     """Same 14 positional arguments as the pybind function.  ``chunk_size`` and ``noop_flag`` are ignored
-    (the reference kernel never reads ``noop_flag``, fused_adam_cuda_kernel.cu:26)."""
+    (the reference kernel never reads ``noop_flag``, fused_adam_cuda_kernel.cu:26).  The kernels index raw memory,
+    so what the reference leaves to asserts is checked here for every tensor: dtype per list, one device, equal sizes."""
+    code = _mode(tensor_lists)
+    dtypes = _DTYPES[code]
     n = len(tensor_lists[0])
+    if any(len(lst) != n for lst in tensor_lists):
+        raise RuntimeError("Size mismatch among tensor lists")  # multi_tensor_apply.cuh:55
+    device = tensor_lists[0][0].device
     rows = (_Tensor * n)()
     for t in range(n):
         cols = [lst[t] for lst in tensor_lists]
         if not all(c.is_contiguous() and c.is_cuda and c.numel() == cols[0].numel() for c in cols):
             raise RuntimeError("tensor lists must hold contiguous device tensors of equal numel")  # multi_tensor_apply.cuh:59-65
+        if not all(c.dtype == d and c.device == device for c, d in zip(cols, dtypes)):
+            raise RuntimeError(f"tensor {t}: every list must hold one dtype ({dtypes}) on one device")
         rows[t].p, rows[t].m, rows[t].v, rows[t].g = (c.data_ptr() for c in cols[:4])
         rows[t].p_copy = cols[4].data_ptr() if len(cols) == 5 else None
         rows[t].numel = cols[0].numel()
-    stream = torch.cuda.current_stream().cuda_stream  # the hipStream_t under ROCm
-    rc = _lib.fsadam_step(rows, n, _mode(tensor_lists), lr, beta1, beta2, eps, grad_scale, optim_scale, decay, step, mode,
+    if found_inf.dtype != _F32 or found_inf.device != device:
+        raise RuntimeError("found_inf must be a float32 tensor on the lists' device")
+    stream = torch.cuda.current_stream(device).cuda_stream  # the hipStream_t under ROCm
+    rc = _lib.fsadam_step(rows, n, code, lr, beta1, beta2, eps, grad_scale, optim_scale, decay, step, mode,
                           bias_correction, found_inf.data_ptr(), stream)
     if rc != 0:
         raise RuntimeError(_lib.fsadam_last_error().decode())

@@ -14,15 +14,20 @@ Deliberate differences, all supersets of the reference behaviour:
   raise it (fused_adam_cuda_kernel.cu:94-105 is the only writer), so they step without a host sync.
   In PURE_FP16 it is cleared only after a step that raised it (a flag read back as 0 is still 0).
   The scale bookkeeping they do every step (adam.py:289-295) is kept.
-* After an overflow m and v are zeroed in place rather than re-allocated (adam.py:285-288), and
-  parameters that never had a gradient keep an empty state instead of a half-initialised one.
+* After an overflow m and v are zeroed in place rather than re-allocated (adam.py:285-288).  Parameters that
+  never had a gradient get zero ``exp_avg``/``exp_avg_sq`` without a ``"step"`` there, as in the reference; should
+  such a parameter receive a gradient later, its counter starts at 0 (the reference raises ``KeyError``).
 * ``load_state_dict`` keeps fp32 ``exp_avg``/``exp_avg_sq`` exact for fp16 parameters (the reference
   round-trips them through fp16, adam.py:176-182).
 * The fp32 master copies of MIXED_PRECISION carry no ``.grad`` (the reference allocates a zero one per
   copy, adam.py:128, and never reads it).
-* ``exp_avg``/``exp_avg_sq`` of a parameter that is a view starting between 128-byte lines (packed into a
-  flat buffer) are views too, 512 elements into a slightly longer allocation at most, so that state and
-  parameter leave their lines at the same element (``zeros_like`` in the reference, adam.py:226-228).
+* ``exp_avg``/``exp_avg_sq`` are laid out like the parameters (``zeros_like`` per parameter in the reference,
+  adam.py:226-228): parameters that are back-to-back views of one buffer (OSS's buckets, oss.py:630-659) get
+  state that is back-to-back views of one buffer too, and so do the fp32 master copies of MIXED_PRECISION; a
+  run that starts between 128-byte lines gets state that starts as many elements past a line.  The native
+  layout then treats each run as one tensor.  The placement is re-established (one copy of the state) after
+  ``load_state_dict`` and after ``optimizer.state[p]`` has been assigned directly, as
+  ``OSS.load_state_dict`` does (oss.py:453-461).
 """
 from __future__ import annotations
 
@@ -60,20 +65,58 @@ _NATIVE_MODE = {
 _MAX_OPTIM_SCALE = 2 ** 16
 
 
-def _state_like(p: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    """Zeros of ``p``'s shape for its exp_avg / exp_avg_sq.  A parameter that starts between cache lines (a
-    view packed into a flat buffer) gets state that starts as many elements past a 1 KiB boundary as the
-    parameter does, modulo 512, inside an allocation 512 elements longer: the native layout then finds ONE
-    head length that puts the parameter's and the state's tiles on line boundaries together; with state
-    on its own boundaries the parameter's stream would stay split across lines."""
-    n = p.numel()
-    if n < 8192 or p.data_ptr() % 128 == 0 or not p.is_contiguous():
-        return torch.zeros_like(p, dtype=dtype)
-    want = (p.data_ptr() // p.element_size()) % 512
-    buf = torch.zeros(n + 512, dtype=dtype, device=p.device)
+_PLACE_MIN = 8192  # shorter runs are left where the allocator puts them (the native layout gives them no head either)
+
+
+def _adjacent_runs(tensors: List[torch.Tensor]) -> List[List[int]]:
+    """Indices of ``tensors`` grouped into maximal runs of consecutive entries that lie back to back in
+    memory (entry k+1 starts at the byte behind entry k's last element)."""
+    runs: List[List[int]] = []
+    end = None
+    for k, t in enumerate(tensors):
+        ptr = t.data_ptr()
+        if end is not None and ptr == end and t.is_contiguous() and t.dtype == tensors[k - 1].dtype and t.device == tensors[k - 1].device:
+            runs[-1].append(k)
+        else:
+            runs.append([k])
+        end = ptr + t.numel() * t.element_size() if t.is_contiguous() else None
+    return runs
+
+
+def _needs_offset(first: torch.Tensor, total: int) -> bool:
+    """A run of ``total`` elements starting at ``first`` whose tiles the native layout moves onto line boundaries
+    by splitting off a head: its other streams must then leave their lines at the same element."""
+    return total >= _PLACE_MIN and first.data_ptr() % 128 != 0
+
+
+def _buffer_placed_like(first: torch.Tensor, total: int, dtype: torch.dtype, zero: bool) -> torch.Tensor:
+    """``total`` elements of ``dtype`` for a stream that accompanies a run starting at ``first``.  A run that
+    starts between cache lines gets a stream that starts as many elements past a 1 KiB boundary as it does,
+    modulo 512, inside an allocation 512 elements longer: the native layout then finds ONE head length that
+    puts the tiles of both on line boundaries."""
+    make = torch.zeros if zero else torch.empty
+    if not _needs_offset(first, total):
+        return make(total, dtype=dtype, device=first.device)
+    want = (first.data_ptr() // first.element_size()) % 512
+    buf = make(total + 512, dtype=dtype, device=first.device)
     have = (buf.data_ptr() // buf.element_size()) % 512
     start = (want - have) % 512
-    return buf[start:start + n].view(p.shape)
+    return buf[start:start + total]
+
+
+def _placed(streams: List[torch.Tensor], likes: List[torch.Tensor]) -> bool:
+    """Do ``streams`` (one per entry of the run ``likes``) already lie back to back, at the run's offset?"""
+    first, total = likes[0], sum(t.numel() for t in likes)
+    end = None
+    for st, like in zip(streams, likes):
+        if not st.is_contiguous() or st.numel() != like.numel() or st.device != like.device:
+            return False
+        if end is not None and st.data_ptr() != end:
+            return False
+        end = st.data_ptr() + st.numel() * st.element_size()
+    if _needs_offset(first, total):
+        return (streams[0].data_ptr() // streams[0].element_size()) % 512 == (first.data_ptr() // first.element_size()) % 512
+    return True
 
 
 class _VersionedState(defaultdict):
@@ -192,12 +235,21 @@ class Adam(torch.optim.Optimizer):
 
     def _build_fp32_params(self, params: Any) -> None:
         """fp32 master copies of fp16 parameters, one group (adam.py:123-153)."""
-        masters = []
-        for p in params:
-            master = torch.nn.Parameter(p.data.float()).to(p.device)
-            # the reference also gives every copy a zero .grad (adam.py:128) that nothing ever reads:
-            # 4 bytes per parameter (6.5 GB on a 1.63e9 shard) that are not spent here
-            masters.append(master)
+        # The reference also gives every copy a zero .grad (adam.py:128) that nothing ever reads: 4 bytes per
+        # parameter (6.5 GB on a 1.63e9 shard) that are not spent here.  Parameters that lie back to back in
+        # one buffer get master copies that do too, so that the native layout can treat the run as one tensor.
+        params = list(params)
+        masters: List[Any] = [None] * len(params)
+        datas = [p.data for p in params]
+        for run in _adjacent_runs(datas):
+            likes = [datas[k] for k in run]
+            flat = _buffer_placed_like(likes[0], sum(t.numel() for t in likes), torch.float32, zero=False)
+            at = 0
+            for k, like in zip(run, likes):
+                view = flat[at:at + like.numel()].view(like.shape)
+                view.copy_(like)
+                masters[k] = torch.nn.Parameter(view)
+                at += like.numel()
         group: Dict[str, Any] = {"params": masters}
         for name, default in self.defaults.items():
             group.setdefault(name, default)
@@ -224,17 +276,24 @@ class Adam(torch.optim.Optimizer):
         super().load_state_dict(state_dict)
         self._optim_scale = state_dict["optim_scale"]  # adam.py:174
         # torch casts floating state to the parameter dtype; take m and v from the saved tensors instead
-        # so that fp32 state of fp16 parameters is restored bit for bit.
-        saved_ids = [pid for g in state_dict["param_groups"] for pid in g["params"]]
-        live = [p for g in self.param_groups for p in g["params"]]
+        # so that fp32 state of fp16 parameters is restored bit for bit, and lay them out like the parameters
+        # (one copy, straight into place).
+        saved_ids = [[pid for pid in g["params"]] for g in state_dict["param_groups"]]
         saved_state = state_dict["state"]
-        for pid, p in zip(saved_ids, live):
-            if pid not in saved_state or p not in self.state:
-                continue
-            for key in ("exp_avg", "exp_avg_sq"):
-                if key in saved_state[pid]:
-                    src = saved_state[pid][key]
-                    self.state[p][key] = src.detach().to(device=p.device, dtype=self.optim_type, copy=True)
+        for gi, (group, ids) in enumerate(zip(self.param_groups, saved_ids)):
+            masters = self.fp32_param_groups[gi]["params"] if self.mixed_precision else None
+            states, likes = [], []
+            for pj, (pid, p) in enumerate(zip(ids, group["params"])):
+                if pid not in saved_state or p not in self.state:
+                    continue
+                like = masters[pj] if masters is not None else p
+                state = self.state[p]
+                for key in ("exp_avg", "exp_avg_sq"):
+                    if key in saved_state[pid]:
+                        state[key] = saved_state[pid][key].detach().to(device=like.device, dtype=self.optim_type)
+                states.append(state)
+                likes.append(like)
+            self._place_state(states, likes, fresh_copy=True)
         self._plans_invalidate()
 
     # ------------------------------------------------------------------ the step
@@ -301,39 +360,39 @@ class Adam(torch.optim.Optimizer):
         step_no = None
         params = group["params"]
         depth = 5 if (mixed or copies is not None) else 4
+        # first pass: who takes part, lazy state (adam.py:223-228; the tensors come from _place_state), counters
+        active: List[int] = []
         for pj, p in enumerate(params):
             grad = p.grad
             if grad is None:
                 states.append(None)
-                outs.append(None)
                 continue
             if grad.is_sparse:
                 raise RuntimeError("FusedAdam does not support sparse gradients, please consider SparseAdam instead")
             state = state_map[p]
-            if len(state) == 0:  # adam.py:223-228
+            if "step" not in state:  # empty, or zeroed by an overflow before its first gradient
                 state["step"] = 0
-                like = masters[pj] if mixed else p
-                state["exp_avg"] = _state_like(like, optim_type)
-                state["exp_avg_sq"] = _state_like(like, optim_type)
-            step_no = state["step"] = state["step"] + 1  # the call uses the last parameter's counter (adam.py:272)
             states.append(state)
+            active.append(pj)
+        likes = [masters[pj] if mixed else params[pj] for pj in active]
+        self._place_state([states[pj] for pj in active], likes)
+        for pj, like in zip(active, likes):
+            p, state = params[pj], states[pj]
+            step_no = state["step"] = state["step"] + 1  # the call uses the last parameter's counter (adam.py:272)
             lists = batches.get(p.device)
             if lists is None:
                 lists = batches[p.device] = [[] for _ in range(depth)]
-            lists[0].append(masters[pj] if mixed else p)
+            lists[0].append(like)
             lists[1].append(state["exp_avg"])
             lists[2].append(state["exp_avg_sq"])
-            lists[3].append(grad)
+            lists[3].append(p.grad)
             if mixed:
                 lists[4].append(p)
-                outs.append(None)
             elif copies is not None:
                 if p not in copies:
                     raise RuntimeError("a parameter with a gradient has no fp16 copy attached")
                 lists[4].append(copies[p])
-                outs.append(copies[p])
-            else:
-                outs.append(None)
+        outs = [copies.get(p) if (copies is not None and not mixed and st is not None) else None for p, st in zip(params, states)]
         caches = self.__dict__.setdefault("_group_cache", {})
         if len(batches) == 1:  # one device: the steady-state walks can take over from the next step on
             device = next(iter(batches))
@@ -343,6 +402,40 @@ class Adam(torch.optim.Optimizer):
         else:
             caches.pop(gi, None)
         return batches, step_no
+
+    def _place_state(self, states: List[dict], likes: List[torch.Tensor], fresh_copy: bool = False) -> None:
+        """Give every state dict its ``exp_avg``/``exp_avg_sq``, laid out like the parameters: each run of
+        parameters that lie back to back in memory gets state that lies back to back, starting as many
+        elements past a cache line as the run does.  Missing tensors are created as zeros (adam.py:226-228);
+        tensors that are there but lie elsewhere (restored from a checkpoint, or assigned to
+        ``optimizer.state[p]`` directly) are copied into place once.  State of another dtype, shape or device
+        is left alone: the checks of the step name it.  ``fresh_copy``: the tensors in ``states`` belong to
+        somebody else (a checkpoint): copy them even where they already lie right."""
+        optim_type = self.optim_type
+        for run in _adjacent_runs(likes):
+            run_likes = [likes[k] for k in run]
+            total = sum(t.numel() for t in run_likes)
+            for key in ("exp_avg", "exp_avg_sq"):
+                have = [states[k].get(key) for k in run]
+                there = [t for t in have if t is not None]
+                if any(t.dtype != optim_type or t.numel() != like.numel() or t.device != like.device
+                       for t, like in zip(have, run_likes) if t is not None):
+                    for k, like in zip(run, run_likes):  # foreign state: only fill the gaps
+                        if states[k].get(key) is None:
+                            states[k][key] = _buffer_placed_like(like, like.numel(), optim_type, zero=True).view(like.shape)
+                        elif fresh_copy:
+                            states[k][key] = states[k][key].clone()
+                    continue
+                if len(there) == len(have) and not fresh_copy and _placed(have, run_likes):
+                    continue
+                flat = _buffer_placed_like(run_likes[0], total, optim_type, zero=len(there) < len(have))
+                at = 0
+                for k, like, old in zip(run, run_likes, have):
+                    view = flat[at:at + like.numel()].view(like.shape)
+                    if old is not None:
+                        view.copy_(old.view(like.shape) if old.is_contiguous() else old.reshape(like.shape))
+                    states[k][key] = view
+                    at += like.numel()
 
     def _steady_group(self, gi: int, group: Dict[str, Any]):
         """The cached view of a group whose every parameter took part in the last general walk, or None
@@ -427,6 +520,35 @@ class Adam(torch.optim.Optimizer):
             st["step"] += 1
         return {device: lists}, taking_part[-1]["step"]
 
+    def _launch_group(self, gi: int, group: Dict[str, Any], native_mode: int, watch_overflow: bool, scale, flags: List[torch.Tensor]) -> None:
+        """Walk one parameter group and enqueue its step (adam.py:202-276); the flags to read back are appended to ``flags``."""
+        beta1, beta2 = group["betas"]
+        bias_correction = 1 if group["bias_correction"] else 0
+        ready = self._gather_native(gi, group, native_mode)
+        if ready is not None:
+            plan, table_changed, step_no = ready
+            flag = None
+            if watch_overflow:
+                flag = self._flag_for(plan.device)
+                flags.append(flag)
+            plan.step_rows(table_changed, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
+                           step_no, self.eps_mode, bias_correction, group["weight_decay"])
+            return
+        batches, step_no = self._gather_fast(gi, group)
+        if batches is None:
+            batches, step_no = self._gather(gi, group)
+        if not batches:
+            # adam.py:256 indexes the first device of an empty dict
+            raise IndexError("list index out of range")
+        for device, lists in batches.items():
+            flag = None
+            if watch_overflow:
+                flag = self._flag_for(device)
+                flags.append(flag)
+            self._plan_for(gi, device, native_mode).step(
+                lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag, step_no, self.eps_mode,
+                bias_correction, group["weight_decay"])
+
     def step(self, closure: Optional[Callable[[], float]] = None, *, scale: Union[float, torch.Tensor] = 1.0) -> Optional[float]:
         """One optimization step (adam.py:184-297).
 
@@ -438,6 +560,14 @@ class Adam(torch.optim.Optimizer):
                 (``clip_grad_norm_(..., fold="device")``) costs no host synchronisation.
         """
         loss = closure() if closure is not None else None
+        # What the native call would refuse is checked before the walk touches a step counter, so that a refused
+        # step leaves the optimizer as it was.  (The reference counts first too, adam.py:234, but its native call
+        # has no such refusals.)
+        if isinstance(scale, torch.Tensor) and (scale.dtype != torch.float32 or scale.numel() != 1 or not scale.is_cuda):
+            raise RuntimeError("a tensor scale must be float32 with one element on the parameters' device")
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("Adam.step() cannot be captured into a graph: the step size depends on the step count and "
+                               "travels by value, so every replay would repeat this step's bias correction")
         self.__dict__.setdefault("_plans", {})  # absent after unpickling
         self.__dict__.setdefault("_flags", {})
         native_mode = _NATIVE_MODE[self.precision]
@@ -446,34 +576,13 @@ class Adam(torch.optim.Optimizer):
         watch_overflow = self.precision is Precision.PURE_FP16
 
         for gi, group in enumerate(self.param_groups):
-            beta1, beta2 = group["betas"]
             flags: List[torch.Tensor] = []
-            bias_correction = 1 if group["bias_correction"] else 0
-            ready = self._gather_native(gi, group, native_mode)
-            if ready is not None:
-                plan, table_changed, step_no = ready
-                flag = None
-                if watch_overflow:
-                    flag = self._flag_for(plan.device)
-                    flags.append(flag)
-                plan.step_rows(table_changed, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
-                               step_no, self.eps_mode, bias_correction, group["weight_decay"])
-                batches = None
+            if torch.autograd._profiler_enabled():
+                # a named range around the walk and the launch, as OSS puts one around its optimizer step (oss.py:230)
+                with torch.autograd.profiler.record_function("fairscale_amd::adam::fused_step"):
+                    self._launch_group(gi, group, native_mode, watch_overflow, scale, flags)
             else:
-                batches, step_no = self._gather_fast(gi, group)
-                if batches is None:
-                    batches, step_no = self._gather(gi, group)
-                if not batches:
-                    # adam.py:256 indexes the first device of an empty dict
-                    raise IndexError("list index out of range")
-            for device, lists in (batches or {}).items():
-                flag = None
-                if watch_overflow:
-                    flag = self._flag_for(device)
-                    flags.append(flag)
-                self._plan_for(gi, device, native_mode).step(
-                    lists, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag, step_no, self.eps_mode,
-                    bias_correction, group["weight_decay"])
+                self._launch_group(gi, group, native_mode, watch_overflow, scale, flags)
 
             overflowed = self._read_flags(flags) if flags else False  # adam.py:278
             if overflowed:
@@ -493,18 +602,22 @@ class Adam(torch.optim.Optimizer):
         return loss
 
     def _zero_all_state(self) -> None:
-        """m = v = 0 for every parameter of every group (adam.py:285-288)."""
+        """m = v = 0 for every parameter of every group (adam.py:285-288): in place where the tensors are
+        there (their layout stays), fresh zeros where they are not -- also for parameters that have not had a
+        gradient yet, which the reference gives state here as well."""
         stale: List[torch.Tensor] = []
+        created = False
         for group in self.param_groups:
             for p in group["params"]:
-                state = self.state.get(p)
-                if not state:
-                    continue
+                state = self.state[p]
                 for key in ("exp_avg", "exp_avg_sq"):
                     t = state.get(key)
                     if t is not None and t.dtype == self.optim_type and t.shape == p.shape and t.device == p.device:
                         stale.append(t)
                     else:
                         state[key] = torch.zeros_like(p, dtype=self.optim_type)
+                        created = True
         if stale:
             torch._foreach_zero_(stale)
+        if created:
+            self._group_cache = {}  # the next step walks the list again and lays the new tensors out with the rest

@@ -79,6 +79,7 @@ typedef struct FsAdamPlanInfo {
     int64_t block;             /* threads per workgroup                                                 */
     int64_t lds_throttle;      /* bytes of LDS ballast per workgroup                                    */
     int64_t uploads;           /* how many times the table has been (re)sent to the device              */
+    int64_t n_runs;            /* rows the layout works on: non-empty tensors after merging (option merge_runs) */
 } FsAdamPlanInfo;
 
 /* How fsadam_plan_set_tensors would cut a tensor list into descriptors (see fsadam_layout). */
@@ -96,6 +97,7 @@ typedef struct FsAdamLayout {
     int64_t n_mid_tensors;       /* mid_chunk_elems <= numel < 131072                                          */
     int64_t n_mid_descriptors;
     int64_t grid_mid;            /* workgroups of the middle-sized tensors                                     */
+    int64_t n_runs;              /* non-empty tensors after merging; the three n_*_tensors above count these    */
 } FsAdamLayout;
 
 /* ---- library ---- */
@@ -112,21 +114,13 @@ const char* fsadam_last_error(void);
 float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_correction);
 
 /* Tuning knobs, by name; returns FSADAM_EINVAL for an unknown name or a value out of range.
- *   "block"         threads per workgroup: 64, 128 or 256 (default 64)
- *   "groups"        vectors per lane per stream: 1 or 2 (default 1)
  *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
  *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
  *                   per-mode default (12-16 KiB, default)
- *   "xcd_remap"     0: tiles in dispatch order (default); R > 0: regroup so that each of the eight XCDs
- *                   takes runs of R consecutive tiles (a very large R gives each XCD one contiguous eighth)
- *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
- *                   4 for one that writes the gradients back (default 0)
- *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
- *   "grad_waves"    gradient pass: tiles (one wave each) per workgroup, 1, 4 or 16; the workgroup writes one
- *                   partial result.  0 = 16 for a read-only pass, 1 for one that writes back (default 0)
- *   "unaligned_vectors"  1 (default): full tiles of a tensor whose streams are only element-aligned (a view that
- *                   starts at an odd element) still move with 64/128-bit vector instructions; 0: such tensors
- *                   are processed element by element (measured 1.5-2x slower)
+ *   "merge_runs"    1 (default): consecutive rows of a list that continue each other in every stream (p, m, v, g and
+ *                   the fp16 copy each start where the row before ended: parameters that are back-to-back views of
+ *                   one buffer, with gradients and state laid out alike) are laid out as ONE tensor, so that a
+ *                   list of views into flat buffers costs what the flat buffers cost; 0: every row on its own
  *   "align_heads"   1 (default): a tensor of 8192 elements or more whose streams start off a 128-byte line (a view
  *                   into a flat buffer) gives its first elements, at most 511, to a short descriptor of their own, so
  *                   that every tile behind them starts on line boundaries (see fsadam_head_elems); 0: tiles start
@@ -138,14 +132,15 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *   "upload_stream" 1 (default): a new descriptor table is copied to the device on a stream the library owns,
  *                   and the caller's stream waits for that copy's event, so the copy overlaps the step still
  *                   running on the caller's stream; 0: the copy is enqueued on the caller's stream
- *   "lazy_events"   0 (default): an event is recorded behind every step (and gradient pass); it is what the library
- *                   waits for before it overwrites a table a step may still read, and what orders a call on
- *                   another stream behind the one before.  1: the event is only recorded when one of those needs
- *                   it, which makes a step 3 us shorter, but touches the stream after the call that used it has
- *                   returned: every stream ever passed must then stay alive until the plan is destroyed (for
- *                   fsadam_step / fsadam_grad_pass: until fsadam_clear_cache)
- *   "max_large_chunk"    upper bound of the elements one shared descriptor of a large tensor covers: a
- *                   power of two in [4096, 2^24] (default 2^24; smaller values measured no faster)
+ *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
+ *                   4 for one that writes the gradients back (default 0)
+ *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
+ *   "grad_waves"    gradient pass: tiles (one wave each) per workgroup, 1, 4 or 16; the workgroup writes one
+ *                   partial result.  0 = 16 for a read-only pass, 1 for one that writes back (default 0)
+ * A workgroup of the step is one wave64 handling one vector per lane and stream, tiles are taken in dispatch order
+ * and full tiles of streams that are only element-aligned use the same vector instructions: the alternatives
+ * (128/256 threads, two vectors per lane, an XCD-aware tile order, element-wise tiles, smaller shared chunks)
+ * were measured no faster or slower and are not offered.
  * Affects plans whose tensors are set after the call. */
 int fsadam_set_option(const char* name, int64_t value);
 int fsadam_get_option(const char* name, int64_t* value);
@@ -186,6 +181,13 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
                      float optim_scale, float decay, int step, int eps_mode, int bias_correction,
                      float* found_inf_dev, void* hip_stream);
 int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out);
+/* on = 0 (default): an event is recorded behind every step of the plan; it is what the library waits for before it
+ * overwrites a table a step may still read, and what orders a call on another stream behind the one before.
+ * on = 1: the event is only recorded when one of those needs it, which makes a step 3 us shorter, but touches the
+ * stream after the call that used it has returned: every stream passed to this plan must then stay alive until
+ * fsadam_plan_destroy.  (The Python binding switches it on for its plans: torch's streams live as long as the
+ * process.  fsadam_step and fsadam_grad_pass always record.) */
+int fsadam_plan_lazy_events(FsAdamPlan* plan, int on);
 int fsadam_plan_destroy(FsAdamPlan* plan);
 
 /* As fsadam_plan_step, with the gradient scale read by the kernel from device memory (one float that must be
@@ -200,7 +202,8 @@ int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float be
 
 /* Host-only planning (no device needed): how the list would be laid out under the current options.
  * tensor_class[n_tensors] (may be NULL): 0 empty, 1 small, 2 large, 3 middle-sized.  vector_ok[n_tensors] (may be
- * NULL): 1 = every stream aligned to its 64/128-bit vector. */
+ * NULL): 1 = every stream aligned to its 64/128-bit vector.  With option merge_runs a tensor is laid out with
+ * the run of consecutive tensors it belongs to: class, alignment and head are the run's. */
 int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mode, FsAdamLayout* out,
                   uint8_t* tensor_class, uint8_t* vector_ok);
 

@@ -8,7 +8,7 @@
  * Prints one line per case and exits 0 when everything is as expected.
  *
  * Built by tests/cabi_driver/Makefile (hipcc as the C compiler driver for the runtime's include and
- * library paths); run by tests/test_cabi_driver_gpu.py.
+ * library paths); run by tests/test_cabi_driver.py.
  */
 #include <hip/hip_runtime_api.h>
 #include <stdint.h>

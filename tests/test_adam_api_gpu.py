@@ -296,7 +296,12 @@ def test_trajectory_matches_oracle_state_machine(oracle, api, cuda_device, preci
                 assert np.array_equal(master.detach().cpu().numpy(), ref.fp32_params[j])
     if mode == PURE16:
         assert opt._optim_scale < 2.0 ** 16 or ref.optim_scale == 2.0 ** 16  # it backed off at step 4 (and may have regrown)
-    assert len(opt.state[params[0]]) == 0  # a parameter that never had a gradient keeps an empty state
+    never = opt.state[params[0]]  # a parameter that never had a gradient
+    if mode == PURE16:  # the overflow of step 4 gave it zero state without a counter, as adam.py:285-288 does
+        assert set(never) == {"exp_avg", "exp_avg_sq"}
+        assert all(not t.any() and t.dtype == torch.float16 and t.shape == params[0].shape for t in never.values())
+    else:
+        assert len(never) == 0
 
 
 @pytest.mark.parametrize("seed", range(10))
@@ -502,6 +507,11 @@ def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_
             at += p.numel()
         for opt in opts:
             opt.step(scale=2.0)
+    # the packed list is ONE run for the native layout (parameters, gradients, state and in MIXED_PRECISION the fp32
+    # master copies all lie back to back); the separately allocated one is five
+    infos = [next(iter(opt._plans.values())).info() for opt in opts]
+    assert 1 < infos[0]["n_runs"] <= len(sizes) and infos[1]["n_runs"] == 1
+    assert infos[1]["n_descriptors"] < infos[0]["n_descriptors"]
     for p, q in zip(separate, packed):
         assert torch.equal(p.detach(), q.detach())
         for key in ("exp_avg", "exp_avg_sq"):
@@ -518,6 +528,292 @@ def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_
     for q in packed:
         for key in ("exp_avg", "exp_avg_sq"):
             assert torch.equal(fresh.state[q][key], opts[1].state[q][key])
+
+
+# ---- runs: parameters that are back-to-back views of one buffer (oss.py:630-659, param_bucket.py:62-90)
+
+def _packed_problem(precision_name, device, sizes, lead=3, seed=5):
+    """The parameters of ``_random_problem`` once separately allocated and once as views packed back to back into a
+    flat buffer that starts ``lead`` elements in, with a flat gradient buffer of the same layout."""
+    separate = _random_problem(precision_name, device, sizes, seed)
+    dtype = separate[0].dtype
+    flat = torch.empty(sum(sizes) + lead, device=device, dtype=dtype)
+    flat_grad = torch.zeros_like(flat)
+    packed, grad_views, at = [], [], lead
+    for p in separate:
+        view = flat[at:at + p.numel()]
+        view.copy_(p.detach())
+        packed.append(view.requires_grad_())
+        grad_views.append(flat_grad[at:at + p.numel()])
+        at += p.numel()
+    return separate, packed, grad_views
+
+
+def _runs(opt):
+    return next(iter(opt._plans.values())).info()["n_runs"]
+
+
+ALL_PRECISIONS = ["FULL_PRECISION", "MIXED_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION", "PURE_FP16"]
+
+
+@pytest.mark.parametrize("precision_name", ALL_PRECISIONS)
+def test_a_stream_that_breaks_the_sequence_splits_the_run(api, cuda_device, precision_name):
+    """Packed parameters whose gradients are NOT all packed: the gradient of the third parameter lives in an
+    allocation of its own, so the list is three runs (before, the odd one, after); a parameter in the middle that
+    gets no gradient (frozen) splits its run as well.  Values as for separately allocated parameters throughout."""
+    Adam, _, Precision = api
+    sizes = (9001, 33, 8192, 140003, 20000, 7)
+    separate, packed, grad_views = _packed_problem(precision_name, cuda_device, sizes)
+    opts = [Adam(ps, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name]) for ps in (separate, packed)]
+    odd = torch.empty(sizes[2], device=cuda_device, dtype=packed[0].dtype)
+    for step in range(1, 7):
+        _set_grads(separate, step)
+        frozen = 4 if step >= 4 else None  # from step 4 on the fifth parameter sits out
+        for j, (p, q, gv) in enumerate(zip(separate, packed, grad_views)):
+            if j == frozen:
+                p.grad = q.grad = None
+            else:
+                q.grad = (odd if j == 2 else gv).copy_(p.grad)
+        for opt in opts:
+            opt.step()
+        # (separately allocated tensors may merge as well, where the allocator happens to put them back to back)
+        assert _runs(opts[0]) <= (len(sizes) if frozen is None else len(sizes) - 1)
+        assert _runs(opts[1]) == (3 if frozen is None else 4), step
+    for p, q in zip(separate, packed):
+        assert torch.equal(p.detach(), q.detach())
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(opts[0].state[p][key], opts[1].state[q][key])
+
+
+@pytest.mark.parametrize("precision_name", ALL_PRECISIONS)
+def test_state_that_does_not_follow_the_parameters_is_put_in_place(api, cuda_device, precision_name):
+    """Gradients and parameters packed, the state not: ``optimizer.state[p]`` assigned directly with tensors
+    allocated one by one (what ``OSS.load_state_dict`` does, oss.py:453-461).  The step after that lays the state
+    out with the parameters again (one copy), the list is one run, and the values go on as if nothing had happened."""
+    Adam, _, Precision = api
+    sizes = (9001, 33, 8192, 140003, 20000)
+    separate, packed, grad_views = _packed_problem(precision_name, cuda_device, sizes)
+    opts = [Adam(ps, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name]) for ps in (separate, packed)]
+
+    def both_step(step):
+        _set_grads(separate, step)
+        for p, q, gv in zip(separate, packed, grad_views):
+            q.grad = gv.copy_(p.grad)
+        for opt in opts:
+            opt.step()
+
+    for step in (1, 2):
+        both_step(step)
+    assert _runs(opts[1]) == 1
+    for q in packed:
+        old = opts[1].state[q]
+        opts[1].state[q] = {"step": old["step"], "exp_avg": old["exp_avg"].clone(), "exp_avg_sq": old["exp_avg_sq"].clone()}
+    strays = [opts[1].state[q]["exp_avg"] for q in packed]
+    for step in (3, 4):
+        both_step(step)
+    assert _runs(opts[1]) == 1
+    assert all(opts[1].state[q]["exp_avg"] is not t for q, t in zip(packed, strays))
+    for p, q in zip(separate, packed):
+        assert torch.equal(p.detach(), q.detach())
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(opts[0].state[p][key], opts[1].state[q][key])
+
+
+# ---- what the callers' checkpoint flows do to this optimizer (done by hand: the callers themselves are out of scope)
+
+def _copy_to_device(value, device):
+    """fairscale.internal.params.recursive_copy_to_device (params.py:29-56) in four lines."""
+    if isinstance(value, torch.Tensor):
+        return value.to(device)
+    if isinstance(value, (list, tuple)):
+        return type(value)(_copy_to_device(v, device) for v in value)
+    if isinstance(value, dict):
+        return {k: _copy_to_device(v, device) for k, v in value.items()}
+    return value
+
+
+def _lock_step(opt_a, params_a, opt_b, params_b, first_step, steps=3, overflow_at=None):
+    for step in range(first_step, first_step + steps):
+        _set_grads(params_a, step)
+        if overflow_at == step:
+            params_a[-1].grad[5] = 6e4
+        for p, q in zip(params_a, params_b):
+            q.grad = p.grad.clone() if q.grad is None or q.grad.data_ptr() == p.grad.data_ptr() else q.grad.copy_(p.grad)
+        opt_a.step()
+        opt_b.step()
+        assert opt_a._optim_scale == opt_b._optim_scale
+        for p, q in zip(params_a, params_b):
+            assert torch.equal(p.detach(), q.detach()), f"step {step}"
+            for key in ("exp_avg", "exp_avg_sq"):
+                assert torch.equal(opt_a.state[p][key], opt_b.state[q][key]), f"step {step} {key}"
+            assert opt_a.state[p]["step"] == opt_b.state[q]["step"]
+
+
+def _clone_problem(params, opt, Adam, precision, packed):
+    """Parameters with the values ``params`` hold now (packed into one buffer or one by one) and a fresh optimizer;
+    in MIXED_PRECISION the fp32 master copies are carried over, as the reference's tests do (test_adam.py:90-95)."""
+    if packed:
+        flat = torch.empty(sum(p.numel() for p in params) + 3, device=params[0].device, dtype=params[0].dtype)
+        flat_grad = torch.zeros_like(flat)
+        clones, at = [], 3
+        for p in params:
+            view = flat[at:at + p.numel()]
+            view.copy_(p.detach())
+            clones.append(view.requires_grad_())
+            clones[-1].grad = flat_grad[at:at + p.numel()]
+            at += p.numel()
+    else:
+        clones = [p.detach().clone().requires_grad_() for p in params]
+    fresh = Adam(clones, lr=1e-2, weight_decay=0.01, precision=precision)
+    if opt.fp32_param_groups:
+        for mine, theirs in zip(fresh.fp32_param_groups[0]["params"], opt.fp32_param_groups[0]["params"]):
+            mine.data.copy_(theirs.data)
+    return clones, fresh
+
+
+@pytest.mark.parametrize("precision_name", ALL_PRECISIONS)
+@pytest.mark.parametrize("packed", [False, True])
+def test_state_moved_to_the_cpu_and_assigned_back_directly_as_oss_does(api, cuda_device, precision_name, packed):
+    """``OSS.consolidate_state_dict`` copies ``optim.state_dict()`` to the CPU recursively (oss.py:333-336);
+    ``OSS.load_state_dict`` copies each parameter's entry back to the device and assigns it to
+    ``optim.state[param]`` directly (oss.py:453-461) -- ``Adam.load_state_dict`` never runs and ``optim_scale``
+    is not part of what OSS saves (oss.py:413).  After that the two optimizers must stay in lock step; in
+    PURE_FP16 that needs the scale the state was stored with, which the caller has to carry over."""
+    Adam, _, Precision = api
+    precision = Precision[precision_name]
+    sizes = (9001, 33, 8192, 140003)
+    params = _random_problem(precision_name, cuda_device, sizes)
+    opt = Adam(params, lr=1e-2, weight_decay=0.01, precision=precision)
+    opt._optim_scale_update_freq = 2  # PURE_FP16: the scale moves during the test
+    for step in range(1, 5):
+        _set_grads(params, step)
+        if precision_name == "PURE_FP16" and step == 3:
+            params[-1].grad[7] = 6e4  # an overflow: the saved scale is not the constructor's
+        opt.step()
+    saved = _copy_to_device(opt.state_dict(), torch.device("cpu"))
+    assert all(t.device.type == "cpu" for st in saved["state"].values() for t in st.values() if isinstance(t, torch.Tensor))
+    clones, fresh = _clone_problem(params, opt, Adam, precision, packed)
+    fresh._optim_scale_update_freq = 2
+    for pid, q in zip(saved["param_groups"][0]["params"], clones):
+        fresh.state[q] = _copy_to_device(saved["state"][pid], q.device)
+    if precision_name == "PURE_FP16":
+        assert saved["optim_scale"] != fresh._optim_scale
+    fresh._optim_scale = saved["optim_scale"]
+    fresh._steps_since_optim_scale_change = opt._steps_since_optim_scale_change
+    _lock_step(opt, params, fresh, clones, first_step=5, steps=4, overflow_at=7 if precision_name == "PURE_FP16" else None)
+    if packed:
+        assert _runs(fresh) == 1  # the directly assigned state was laid out with the packed parameters
+
+
+@pytest.mark.parametrize("precision_name", ALL_PRECISIONS)
+def test_state_of_a_flat_parameter_cut_into_slices_and_flattened_again_as_fsdp_does(api, cuda_device, precision_name):
+    """FSDP's full optimizer state dict holds, per original parameter, the slice of the flat parameter's state
+    viewed in that parameter's shape (``_unflatten_optim_state``, fsdp_optim_utils.py:120-200) and ``step`` once;
+    loading flattens again with ``torch.cat`` of the reshaped slices (``flatten_optim_state_dict``, :38-52) and
+    hands the result to ``optim.load_state_dict``."""
+    Adam, _, Precision = api
+    precision = Precision[precision_name]
+    shapes = [(50, 100), (4000,), (3, 7, 11), (130000,)]
+    numels = [int(np.prod(sh)) for sh in shapes]
+    flat = _random_problem(precision_name, cuda_device, (sum(numels),))
+    opt = Adam(flat, lr=1e-2, weight_decay=0.01, precision=precision)
+    for step in range(1, 4):
+        _set_grads(flat, step)
+        opt.step()
+    sd = _copy_to_device(opt.state_dict(), torch.device("cpu"))
+    # unflatten: one entry per original parameter
+    unflat = {}
+    for gid, (n, sh, start) in enumerate(zip(numels, shapes, np.cumsum([0] + numels[:-1]))):
+        unflat[gid] = {key: sd["state"][0][key][start:start + n].clone().view(sh) for key in ("exp_avg", "exp_avg_sq")}
+        unflat[gid]["step"] = sd["state"][0]["step"]
+    assert [tuple(unflat[g]["exp_avg"].shape) for g in unflat] == shapes
+    # flatten again
+    again = {"state": {0: {key: torch.cat([unflat[g][key].reshape(-1) for g in sorted(unflat)]) for key in ("exp_avg", "exp_avg_sq")}},
+             "param_groups": sd["param_groups"], "optim_scale": sd["optim_scale"]}
+    again["state"][0]["step"] = unflat[0]["step"]
+    clones, fresh = _clone_problem(flat, opt, Adam, precision, packed=False)
+    fresh.load_state_dict(again)
+    assert fresh.state[clones[0]]["exp_avg"].dtype == opt.optim_type and fresh.state[clones[0]]["exp_avg"].is_cuda
+    _lock_step(opt, flat, fresh, clones, first_step=4)
+
+
+@pytest.mark.parametrize("precision_name", ALL_PRECISIONS)
+def test_load_state_dict_lays_the_state_out_with_packed_parameters(api, cuda_device, precision_name):
+    """A checkpoint written by an optimizer over separately allocated parameters, loaded by one over packed
+    views: the restored state is packed like the parameters (the list is one run from the first step on, without
+    a second copy), bit for bit what was saved, and the two stay in lock step."""
+    Adam, _, Precision = api
+    precision = Precision[precision_name]
+    params = _random_problem(precision_name, cuda_device, (9001, 33, 8192, 140003))
+    opt = Adam(params, lr=1e-2, weight_decay=0.01, precision=precision)
+    for step in range(1, 4):
+        _set_grads(params, step)
+        opt.step()
+    blob = io.BytesIO()
+    torch.save(opt.state_dict(), blob)
+    blob.seek(0)
+    clones, fresh = _clone_problem(params, opt, Adam, precision, packed=True)
+    fresh.load_state_dict(torch.load(blob, weights_only=True))
+    states = [fresh.state[q]["exp_avg"] for q in clones]
+    for a, b in zip(states, states[1:]):
+        assert b.data_ptr() == a.data_ptr() + a.numel() * a.element_size()
+    _lock_step(opt, params, fresh, clones, first_step=4)
+    assert _runs(fresh) == 1
+    assert all(fresh.state[q]["exp_avg"] is t for q, t in zip(clones, states)), "the loaded state was copied a second time"
+
+
+def test_a_table_the_library_refused_is_sent_again(api, cuda_device, monkeypatch):
+    """When ``fsadam_plan_set_tensors`` fails after the gradients have moved (out of memory for the table, a HIP
+    error), the row buffer already holds the new pointers.  The next step must not take 'nothing changed' for
+    'the device table is current': it sends the table again and the results are those of an undisturbed run."""
+    from fairscale_amd import _cabi
+
+    Adam, _, _ = api
+    a = _random_problem("FULL_PRECISION", cuda_device, sizes=(1000, 70001), seed=21)
+    b = [p.detach().clone().requires_grad_() for p in a]
+    opt_a, opt_b = Adam(a, lr=1e-2), Adam(b, lr=1e-2)
+    for step in (1, 2):
+        _set_grads(a, step, seed=21)
+        _set_grads(b, step, seed=21)
+        opt_a.step()
+        opt_b.step()
+    plan = next(iter(opt_b._plans.values()))
+    assert plan.info()["uploads"] == 2  # _set_grads makes new tensors: the pointers move every step
+    L = _cabi.lib()
+    real = L.fsadam_plan_set_tensors
+    calls = []
+
+    class Once:
+        def __call__(self, *args):
+            calls.append(1)
+            if len(calls) == 1:
+                return -3  # FSADAM_ENOMEM, nothing was done
+            return real(*args)
+
+    _set_grads(a, 3, seed=21)
+    _set_grads(b, 3, seed=21)
+    monkeypatch.setattr(L, "fsadam_plan_set_tensors", Once())
+    with pytest.raises(_cabi.FsAdamError):
+        opt_b.step()
+    # The training loop catches the error and steps again with the same gradients (which have not moved this time).
+    # The refused step had advanced b's counters (the walk runs before the native call); a is put in the same place.
+    for p in a:
+        opt_a.state[p]["step"] += 1
+    opt_a.step()
+    opt_b.step()
+    monkeypatch.undo()
+    assert len(calls) == 3 and plan.info()["uploads"] == 3  # refused for b, then a, then b again: the table was re-sent
+    for step in (4, 5):
+        _set_grads(a, step, seed=21)
+        _set_grads(b, step, seed=21)
+        opt_a.step()
+        opt_b.step()
+    torch.cuda.synchronize(cuda_device)
+    for p, q in zip(a, b):
+        assert opt_a.state[p]["step"] == opt_b.state[q]["step"] == 6
+        assert torch.equal(p.detach(), q.detach())
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(opt_a.state[p][key], opt_b.state[q][key])
 
 
 def test_hyperparameters_left_as_numpy_scalars_or_tensors_are_accepted(api, cuda_device):
@@ -685,13 +981,13 @@ def test_a_step_on_a_capturing_stream_is_refused(api, cuda_device):
     torch.cuda.synchronize(cuda_device)
     before = [p.detach().clone() for p in params]
     graph = torch.cuda.CUDAGraph()
-    with pytest.raises(RuntimeError, match="captured"):
+    with pytest.raises(RuntimeError, match="captured"):  # raised by Adam.step before anything is touched
         with torch.cuda.graph(graph):
             opt.step()
     torch.cuda.synchronize(cuda_device)
     for p, b in zip(params, before):
         assert torch.equal(p, b)
-    assert opt.state[params[0]]["step"] == 2  # the walk had advanced the counters before the native call refused
+    assert opt.state[params[0]]["step"] == 1  # refused before the walk: no counter moved
     opt.step()
     torch.cuda.synchronize(cuda_device)
     assert not torch.equal(params[1], before[1])

@@ -74,19 +74,21 @@ def test_step_size_is_bit_identical_to_the_oracle(oracle):
 
 
 def test_options_roundtrip_and_validation():
-    old = {k: _cabi.get_option(k) for k in ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "grad_waves", "grad_items",
-                                                "grad_lds_throttle", "unaligned_vectors", "align_heads", "lazy_events", "mid_tiles", "upload_stream")}
+    names = ("lds_throttle", "grad_waves", "grad_items", "grad_lds_throttle", "align_heads", "merge_runs", "mid_tiles", "upload_stream")
+    old = {k: _cabi.get_option(k) for k in names}
+    assert old == {"lds_throttle": -1, "grad_waves": 0, "grad_items": 0, "grad_lds_throttle": -1, "align_heads": 1, "merge_runs": 1,
+                   "mid_tiles": 16, "upload_stream": 1}
     try:
-        _cabi.set_option("block", 128)
-        _cabi.set_option("groups", 2)
         _cabi.set_option("lds_throttle", 20480)
-        assert (_cabi.get_option("block"), _cabi.get_option("groups"), _cabi.get_option("lds_throttle")) == (128, 2, 20480)
-        for flag in ("align_heads", "lazy_events", "upload_stream"):
+        assert _cabi.get_option("lds_throttle") == 20480
+        for flag in ("align_heads", "merge_runs", "upload_stream"):
             for value in (0, 1):
                 _cabi.set_option(flag, value)
                 assert _cabi.get_option(flag) == value
-        for name, bad in (("block", 96), ("groups", 3), ("lds_throttle", 1 << 20), ("xcd_remap", -1), ("max_large_chunk", 5000), ("max_large_chunk", 2048), ("grad_waves", 3), ("grad_items", 5), ("unaligned_vectors", 2),
-                          ("align_heads", 2), ("lazy_events", -1), ("mid_tiles", 3), ("mid_tiles", 128), ("upload_stream", 2), ("no_such_option", 1)):
+        for name, bad in (("lds_throttle", 1 << 20), ("grad_waves", 3), ("grad_items", 5), ("align_heads", 2), ("merge_runs", -1), ("mid_tiles", 3),
+                          ("mid_tiles", 128), ("upload_stream", 2), ("no_such_option", 1),
+                          # shapes and orders that were measured and dropped are not options any more
+                          ("block", 64), ("groups", 1), ("xcd_remap", 0), ("max_large_chunk", 65536), ("unaligned_vectors", 1), ("lazy_events", 1)):
             with pytest.raises(_cabi.FsAdamError):
                 _cabi.set_option(name, bad)
     finally:
@@ -106,10 +108,8 @@ def layout(tensors, mode):
 def test_layout_classes_and_descriptor_counts():
     A = 0x7000_0000_0000  # fake, 2 MiB-aligned device addresses: never dereferenced on the host
     t = lambda n, off=0: (A + off, A + (1 << 32), A + (2 << 32), A + (3 << 32) + off, 0, n)  # noqa: E731
-    old = {k: _cabi.get_option(k) for k in ("block", "groups", "mid_tiles")}
+    old = {k: _cabi.get_option(k) for k in ("mid_tiles",)}
     try:
-        _cabi.set_option("block", 64)
-        _cabi.set_option("groups", 1)
         _cabi.set_option("mid_tiles", 0)  # two classes: shared descriptors from 131072 elements, one per tile below
         lay, cls, vec = layout([t(0), t(1), t(255), t(256), t(257), t(131071), t(131072), t(131073), t(1 << 20)], _cabi.FULL_PRECISION)
         assert lay["tile_elems"] == 256  # 64 lanes x 4 fp32
@@ -140,10 +140,6 @@ def test_layout_classes_and_descriptor_counts():
         # PURE_FP16 moves 8 halves per lane
         lay, _, _ = layout([t(5000)], _cabi.PURE_FP16)
         assert lay["tile_elems"] == 512 and lay["n_small_descriptors"] == 10
-        _cabi.set_option("block", 256)
-        _cabi.set_option("groups", 2)
-        lay, _, _ = layout([t(5000)], _cabi.FULL_PRECISION)
-        assert lay["tile_elems"] == 2048 and lay["n_small_descriptors"] == 3
     finally:
         for k, v in old.items():
             _cabi.set_option(k, v)
@@ -236,6 +232,59 @@ def test_no_other_head_would_align_better():
         assert (cost(got), got) == (cost(best), best), (case, mode, [hex(s[0]) for s in streams], got, best)
 
 
+def test_rows_that_continue_each_other_are_laid_out_as_one_run():
+    """Back-to-back views of flat buffers (every stream of row t+1 starts where row t's ended) become one run; a
+    stream that breaks the sequence, in any of the lists, starts a new one (fake addresses, host-side planning)."""
+    A = 0x7000_0000_0000
+    sizes = [1000, 3, 70000, 0, 5000, 140000, 9]
+
+    def packed(mode, breaks=(), sizes=sizes):
+        """Rows packed into four (five) flat buffers; `breaks`: (row, stream) pairs where that stream skips 64 bytes."""
+        ps, ss, gs = (2 if mode in (_cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16) else 4,
+                      2 if mode == _cabi.PURE_FP16 else 4, 4 if mode == _cabi.FULL_PRECISION else 2)
+        at = [A, A + (1 << 36), A + (2 << 36), A + (3 << 36), A + (4 << 36)]
+        width = [ps, ss, ss, gs, 2]
+        out = []
+        for t, n in enumerate(sizes):
+            for k in range(5):
+                if (t, k) in breaks:
+                    at[k] += 64
+            out.append((at[0], at[1], at[2], at[3], at[4] if mode == _cabi.MIXED_PRECISION else 0, n))
+            for k in range(5):
+                at[k] += n * width[k]
+        return out
+
+    total = sum(sizes)
+    for mode in (_cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16):
+        tile = 512 if mode == _cabi.PURE_FP16 else 256
+        lay, cls, vec = layout(packed(mode), mode)
+        assert lay["n_runs"] == 1 and lay["n_empty_tensors"] == 1, mode
+        assert cls == [2, 2, 2, 0, 2, 2, 2] and vec == [1, 1, 1, 0, 1, 1, 1]
+        assert lay["n_large_tensors"] == 1 and lay["n_small_tensors"] == 0 and lay["n_mid_tensors"] == 0
+        assert lay["n_large_descriptors"] == -(-total // lay["large_chunk_elems"]) and lay["n_small_descriptors"] == 0
+        assert lay["grid_large"] * tile >= total
+        # the same rows one by one
+        old = _cabi.get_option("merge_runs")
+        try:
+            _cabi.set_option("merge_runs", 0)
+            lay0, cls0, _ = layout(packed(mode), mode)
+        finally:
+            _cabi.set_option("merge_runs", old)
+        assert lay0["n_runs"] == 6 and cls0[3] == 0 and cls0[1] == 1 and cls0[5] == 2
+        # a break in one stream only: p (0), v (2), g (3), and in MIXED the fp16 copy (4)
+        for stream in (0, 2, 3) + ((4,) if mode == _cabi.MIXED_PRECISION else ()):
+            lay, cls, _ = layout(packed(mode, breaks={(4, stream)}), mode)
+            assert lay["n_runs"] == 2, (mode, stream)
+            assert cls[:3] == [3, 3, 3] and cls[4:] == [2, 2, 2]  # 71003 elements in front, 145009 behind
+        # a break at every row: nothing to merge
+        lay, _, _ = layout(packed(mode, breaks={(t, 1) for t in range(1, 7)}), mode)
+        assert lay["n_runs"] == 6
+    # the copy stream of the 4-list modes is not looked at
+    rows4 = packed(_cabi.FULL_PRECISION)
+    rows4 = [r[:4] + (0x1234560 + 8 * i,) + r[5:] for i, r in enumerate(rows4)]
+    assert layout(rows4, _cabi.FULL_PRECISION)[0]["n_runs"] == 1
+
+
 def test_layout_counts_heads_among_the_small_descriptors(two_classes):
     A = 0x7000_0000_0000
     t = lambda n, off: (A + off, A + (1 << 34) + off, A + (2 << 34) + off, A + (3 << 34) + off, 0, n)  # noqa: E731
@@ -268,15 +317,13 @@ def test_layout_matches_a_python_model_on_drawn_lists():
 
     rng = random.Random(42)
     A = 0x7000_0000_0000
-    names = ("block", "groups", "max_large_chunk", "mid_tiles")
+    names = ("mid_tiles",)
     old = {k: _cabi.get_option(k) for k in names}
     try:
         for _ in range(120):
-            block, groups = rng.choice([64, 128, 256]), rng.choice([1, 2])
-            cap = rng.choice([1 << 24, 1 << 16, 1 << 14, 4096])
+            block, groups, cap = 64, 1, 1 << 24
             mid_tiles = rng.choice([0, 1, 2, 16, 16, 64])
-            for k, v in zip(names, (block, groups, cap, mid_tiles)):
-                _cabi.set_option(k, v)
+            _cabi.set_option("mid_tiles", mid_tiles)
             mode = rng.choice([_cabi.FULL_PRECISION, _cabi.MIXED_PRECISION, _cabi.MEMORY_EFFICIENT_MIXED_PRECISION, _cabi.PURE_FP16])
             sizes = [rng.choice([0, 1, rng.randrange(2, 5000), rng.randrange(5000, 131072), 131072, rng.randrange(131072, 1 << 22),
                                  rng.randrange(1 << 22, 1 << 31)]) for _ in range(rng.randrange(1, 30))]

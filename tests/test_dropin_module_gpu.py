@@ -65,3 +65,30 @@ def test_drop_in_raises_runtime_error_like_torch_check(dropin, cuda_device):
         dropin.adam(0, None, [mk(4, 5), mk(4, 6), mk(4, 5), mk(4, 5)], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)
     with pytest.raises(RuntimeError, match="eps_mode"):
         dropin.adam(0, None, [mk(4)] * 4, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 7, 1, 0.0)
+
+
+def test_drop_in_refuses_lists_of_the_wrong_element_type(dropin, cuda_device):
+    """What the reference leaves to asserts that a release build compiles out (fused_adam_cuda_kernel.cu:167-199) is
+    refused on the host, for every tensor, before anything is launched: a kernel would otherwise read the buffers at
+    another element width, past their end."""
+    f32 = lambda *ns: [torch.ones(n, device=cuda_device) for n in ns]  # noqa: E731
+    f16 = lambda *ns: [torch.ones(n, device=cuda_device, dtype=torch.float16) for n in ns]  # noqa: E731
+    flag = torch.zeros(1, device=cuda_device)
+    args = (1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)
+    bad_lists = [
+        [f32(8), f32(8), f32(8), f16(8)],              # fp32 parameters with fp16 gradients in four lists
+        [f32(8), f32(8), f32(8), f32(8), f16(8)],      # five lists with fp32 gradients
+        [f32(8), f32(8), f32(8), f16(8), f32(8)],      # copy-out that is not fp16
+        [f16(8), f32(8), f16(8), f16(8)],              # m and v of different types
+        [f32(8, 8), f32(8, 8), f32(8, 8), f32(8) + f16(8)],  # a later tensor of another type
+        [f32(8), f32(8), f32(8)],                      # three lists
+        [f32(8, 8), f32(8), f32(8, 8), f32(8, 8)],     # lists of different lengths
+    ]
+    for lists in bad_lists:
+        before = [t.clone() for lst in lists for t in lst]
+        with pytest.raises(RuntimeError):
+            dropin.adam(0, None, lists, *args)
+        torch.cuda.synchronize(cuda_device)
+        assert all(torch.equal(a, b) for a, b in zip(before, [t for lst in lists for t in lst]))
+    with pytest.raises(RuntimeError, match="found_inf"):
+        dropin.adam(0, None, [f32(8)] * 4, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag.double(), 1, 1, 1, 0.0)

@@ -67,6 +67,35 @@ def test_oracle_flags_non_finite_like_torch(dtype, bad):
         assert np.isinf(ss) and np.isinf(mx)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("inv_scale", [np.inf, -np.inf, np.nan])
+@pytest.mark.parametrize("with_zero", [True, False])
+def test_oracle_follows_torch_for_a_scale_that_is_not_finite(dtype, inv_scale, with_zero):
+    """A degenerate factor: every finite non-zero gradient becomes an infinity (or NaN), and a gradient that is
+    exactly zero becomes NaN (0 * inf), so the largest stored magnitude is NOT the image of the largest incoming
+    one.  No flag: the incoming values are finite."""
+    grads = _grads(dtype, 3)
+    if with_zero:
+        grads[2][17] = 0.0
+    else:
+        for g in grads:
+            g[g == 0] = 1e-3
+    tg = [torch.from_numpy(g.copy()) for g in grads]
+    found = torch.zeros(1)
+    torch._amp_foreach_non_finite_check_and_unscale_(tg, found, torch.tensor([inv_scale], dtype=torch.float32))
+    f, ss, mx = G.grad_pass_numpy(grads, inv_scale, write_back=True)
+    assert f == found.item() == 0.0
+    for a, b in zip(grads, tg):
+        assert np.array_equal(np.isnan(a), np.isnan(b.numpy())) and np.array_equal(a[~np.isnan(a)], b.numpy()[~np.isnan(a)])
+    want_max = max(t.abs().max().item() for t in tg)  # Python's max keeps the first NaN it is given first; look at all
+    any_nan = any(bool(torch.isnan(t).any()) for t in tg)
+    if any_nan:
+        assert np.isnan(mx) and np.isnan(ss)
+        assert with_zero or np.isnan(inv_scale)
+    else:
+        assert np.isinf(mx) and np.isinf(ss) and np.isinf(want_max)
+
+
 def test_oracle_leaves_gradients_alone_without_write_back():
     grads = _grads(np.float16, 3, scale=256.0)
     before = [g.copy() for g in grads]

@@ -172,6 +172,25 @@ def test_ragged_list_matches_oracle(cuda_device, dtype, inv_scale, write_back):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("inv_scale", [np.inf, -np.inf, np.nan])
+@pytest.mark.parametrize("write_back", [True, False])
+def test_a_scale_that_is_not_finite_follows_torch(cuda_device, dtype, inv_scale, write_back):
+    """With an infinite factor a zero gradient stores NaN (0 * inf) while the largest one stores an infinity: the
+    maximum is NaN as torch's ``abs().max()`` makes it, although the kernel forms the stored maximum from the largest
+    incoming magnitude; without a zero it is an infinity.  From the host and from the device."""
+    for with_zero in (True, False):
+        for on_device in (False, True):
+            host = host_grads(dtype, 12, [5, 4099, 70001])
+            for h in host:
+                h[h == 0] = 1e-3
+            if with_zero:
+                host[2][40000] = 0.0
+            dev, stats, want = run_both(host, cuda_device, float(inv_scale), write_back, scale_on_device=on_device)
+            assert np.isnan(want[2]) == (with_zero or np.isnan(inv_scale))
+            check(host, dev, stats, want, f"{np.dtype(dtype)} inv={inv_scale} zero={with_zero} device={on_device}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_misaligned_views_and_device_resident_scale(cuda_device, dtype):
     host = host_grads(dtype, 11, [5, 4099, 70001, 140001], scale=64.0)
     dev, stats, want = run_both(host, cuda_device, 1 / 64, True, misalign=1, scale_on_device=True)

@@ -226,8 +226,6 @@ def test_power_of_two_grad_scale_is_bitwise_equivariant(oracle):
     c = _run(oracle, MIXED, p0, g16, grad_scale=1.0, **HY)
     d = _run(oracle, MIXED, p0, [(g.astype(np.float32) * 1024).astype(np.float16) for g in g16], grad_scale=1024.0, **HY)
     # halves that are subnormal at scale 1 gain precision at scale 1024: compare where the unscaled half is normal
-    for x, y in zip(c[:4], d[:4]):
-        assert np.array_equal(x.view(np.uint8), y.view(np.uint8)) or True
     normal = np.all([np.abs(g.astype(np.float32)) >= 6.2e-5 for g in g16], axis=0)
     assert normal.sum() > n // 2
     for x, y in zip(c[:4], d[:4]):

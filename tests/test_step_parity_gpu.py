@@ -137,20 +137,12 @@ def test_non_power_of_two_scales(oracle, cuda_device, mode):
 
 @pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
 @pytest.mark.parametrize("which", ["p", "g", "m", "all"])
-@pytest.mark.parametrize("unaligned_vectors", [1, 0])
-def test_misaligned_views(oracle, cuda_device, mode, which, unaligned_vectors):
-    """Views that start 1 element (p: 3) into an allocation, like OSS bucket views.  By default their full
-    tiles still use vector instructions (at element-aligned addresses); with the option off the whole
-    tensor goes down the element-wise path.  Results must not change either way."""
-    from fairscale_amd import _cabi
-
+def test_misaligned_views(oracle, cuda_device, mode, which):
+    """Views that start 1 element (p: 3) into an allocation, like OSS bucket views: their full tiles use
+    the same vector instructions, at element-aligned addresses."""
     mis = {"p": {"p": 3}, "g": {"g": 1}, "m": {"m": 1}, "all": {"p": 1, "g": 1, "m": 1, "v": 1, "p16": 1}}[which]
-    _cabi.set_option("unaligned_vectors", unaligned_vectors)
-    try:
-        run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000, 140001], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
-                 grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
-    finally:
-        _cabi.set_option("unaligned_vectors", 1)
+    run_case(oracle, cuda_device, mode, [5, 4099, 16385, 40000, 140001], 2, 4200 + mode, dict(DEFAULT, decay=0.01),
+             grad_scale=1.0 if mode == FULL else 128.0, misalign=mis, optim_scale=65536.0 if mode == PURE16 else 1.0)
 
 
 @pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
@@ -278,7 +270,7 @@ def options():
     """Set tuning options for one test and put the defaults back afterwards."""
     from fairscale_amd import _cabi
 
-    names = ("block", "groups", "lds_throttle", "xcd_remap", "max_large_chunk", "unaligned_vectors", "lazy_events", "mid_tiles", "upload_stream")
+    names = ("lds_throttle", "mid_tiles", "upload_stream", "align_heads", "merge_runs")
     old = {k: _cabi.get_option(k) for k in names}
 
     def set_many(**kw):
@@ -290,21 +282,8 @@ def options():
         _cabi.set_option(k, v)
 
 
-@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
-@pytest.mark.parametrize("block,groups", [(64, 2), (128, 1), (128, 2), (256, 1), (256, 2)])
-def test_every_compiled_tile_shape_matches_the_oracle(oracle, cuda_device, options, mode, block, groups):
-    """The library is built with six workgroup shapes per mode; the default is one wave and one vector per
-    stream.  The others are reachable through the options and must give the same bits."""
-    options(block=block, groups=groups)
-    tile = block * (8 if mode == PURE16 else 4) * groups
-    sizes = [1, tile - 1, tile, tile + 1, 3 * tile + 5, 131072, 131073, 300001]
-    run_case(oracle, cuda_device, mode, sizes, 2, 4800 + mode, dict(DEFAULT, decay=0.01), grad_scale=1.0 if mode == FULL else 8.0,
-             optim_scale=65536.0 if mode == PURE16 else 1.0, misalign={"p": 1})
-
-
-@pytest.mark.parametrize("setting", [dict(xcd_remap=1), dict(xcd_remap=7), dict(xcd_remap=1 << 20), dict(lds_throttle=0),
-                                     dict(lds_throttle=65536), dict(max_large_chunk=4096), dict(max_large_chunk=65536, block=256, groups=2),
-                                     dict(mid_tiles=0), dict(mid_tiles=2), dict(mid_tiles=64), dict(mid_tiles=4, block=128, xcd_remap=3)])
+@pytest.mark.parametrize("setting", [dict(lds_throttle=0), dict(lds_throttle=65536), dict(mid_tiles=0), dict(mid_tiles=2), dict(mid_tiles=64),
+                                     dict(mid_tiles=4, align_heads=0), dict(merge_runs=0)])
 def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, options, setting):
     options(**setting)
     for mode in (MEMEFF, PURE16):
@@ -316,19 +295,19 @@ def test_launch_geometry_options_do_not_change_results(oracle, cuda_device, opti
 @pytest.mark.parametrize("upload_stream", [1, 0])
 def test_event_bookkeeping_eager_and_lazy(oracle, cuda_device, options, lazy_events, upload_stream):
     """The event behind a step is what protects a table that may still be read and what orders a step on
-    another stream behind the one before.  Recorded behind every step (the library's default) or only when
-    needed (what this package switches on, torch's streams being immortal), the results are the same:
+    another stream behind the one before.  Recorded behind every step (a plan's default) or only when
+    needed (what this package switches on for its plans, torch's streams being immortal), the results are the same:
     steps hopping between three streams without any synchronisation by the caller, with the gradient
     pointers moving every step (a new table every step, the ring of slots wrapping around).  The tables
     travel on a stream of the library's own (default) or on the caller's."""
     from fairscale_amd import fused_adam_hip
 
-    options(lazy_events=lazy_events, upload_stream=upload_stream)
+    options(upload_stream=upload_stream)
     host = C.Tensors(FULL, [5, 4099, 140001, 70000], 5100)
     dev = GpuList(host, cuda_device)
     streams = [torch.cuda.Stream(cuda_device) for _ in range(3)]
     flag = np.zeros(1, np.float32)
-    plan = fused_adam_hip.TensorListPlan(FULL, cuda_device)
+    plan = fused_adam_hip.TensorListPlan(FULL, cuda_device, lazy_events=bool(lazy_events))
     keep = []
     for step in range(1, 13):
         grads = host.grads(step)
@@ -600,11 +579,14 @@ def test_pure_fp16_flag_for_every_position_in_a_vector(oracle, cuda_device, misa
         assert nonfinite == (pos is not None)
 
 
-def test_flat_vs_split_is_bitwise_identical(cuda_device):
+@pytest.mark.parametrize("merge_runs", [0, 1])
+def test_flat_vs_split_is_bitwise_identical(cuda_device, options, merge_runs):
     """Chunking/table invariance at a size the oracle is not needed for: one flat 2^24+5 tensor and
-    the same memory stepped as 7 uneven tensors give identical bits (elementwise path)."""
+    the same memory stepped as 7 uneven tensors give identical bits (elementwise path).  With the rows laid
+    out one by one (merge_runs=0) and, the default, merged back into the one run they form."""
     from fairscale_amd import fused_adam_hip
 
+    options(merge_runs=merge_runs)
     n = (1 << 24) + 5
     gen = torch.Generator(device=cuda_device).manual_seed(7)
     base = [torch.randn(n, device=cuda_device, generator=gen) * s for s in (0.02, 1e-3, 1e-6, 1e-3)]
@@ -618,11 +600,77 @@ def test_flat_vs_split_is_bitwise_identical(cuda_device):
     fused_adam_hip.adam(65536, None, lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 5, 1, 1, 0.01)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+    plan = fused_adam_hip.TensorListPlan(FULL, cuda_device)
+    plan.step(lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 6, 1, 1, 0.01)
+    assert plan.info()["n_runs"] == (1 if merge_runs else 7) and plan.info()["n_tensors"] == 7
+    plan.close()
     # and determinism: the same call on the same inputs twice
     c = [t.clone() for t in base]
     fused_adam_hip.adam(65536, None, [[t] for t in c], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 5, 1, 1, 0.01)
     for x, y in zip(a, c):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+@pytest.mark.parametrize("lead", [0, 3])
+def test_lists_packed_into_flat_buffers_match_the_oracle(oracle, cuda_device, mode, lead):
+    """Every stream of the list packed back to back into a flat buffer of its own (``lead`` elements in), so that the
+    whole list is one run; then the same with the second moment of one tensor and the gradient of another in
+    allocations of their own, which cuts the list into five runs.  Against the oracle, which knows nothing of runs."""
+    from fairscale_amd import fused_adam_hip
+
+    sizes = [5, 4099, 16385, 40000, 140001, 3, 70000]
+    total = sum(sizes)
+    for stray in ({}, {"v": 2, "g": 4}):
+        host = C.Tensors(mode, sizes, 5300 + mode)
+        pd, gd, sd = C.MODE_DTYPES[mode]
+
+        def pack(arrs, name, dtype):
+            flat = torch.empty(total + lead, dtype=TORCH_DTYPE[np.dtype(dtype)], device=cuda_device)
+            out, at = [], lead
+            for i, a in enumerate(arrs):
+                view = flat[at:at + a.size] if stray.get(name) != i else torch.empty(a.size, dtype=flat.dtype, device=cuda_device)
+                view.copy_(torch.from_numpy(a))
+                out.append(view)
+                at += a.size
+            return out
+
+        dev = GpuList.__new__(GpuList)
+        dev.mode, dev.device, dev.misalign = mode, cuda_device, {}
+        dev.p, dev.m, dev.v = pack(host.p, "p", host.p[0].dtype), pack(host.m, "m", sd), pack(host.v, "v", sd)
+        dev.p16 = pack(host.p16, "p16", np.float16) if host.p16 is not None else None
+        dev.found_inf = torch.zeros(1, dtype=torch.float32, device=cuda_device)
+        plan = fused_adam_hip.TensorListPlan(mode, cuda_device)
+        flag = np.zeros(1, np.float32)
+        gs = 1.0 if mode == FULL else 64.0
+        for step in (1, 2):
+            grads = host.grads(step, scale=gs)
+            g = pack(grads, "g", gd)
+            lists = [dev.p, dev.m, dev.v, g] + ([dev.p16] if mode == MIXED else [])
+            kw = dict(DEFAULT, decay=0.01, step=step, grad_scale=gs, optim_scale=65536.0 if mode == PURE16 else 1.0)
+            plan.step(lists, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], gs, kw["optim_scale"], dev.found_inf, step, 1, 1, kw["decay"])
+            torch.cuda.synchronize(cuda_device)
+            oracle_step(oracle, host, grads, flag, **kw)
+            compare(host, dev, f"packed mode={mode} lead={lead} stray={stray} step={step}")
+            assert plan.info()["n_runs"] == (5 if stray else 1)  # [0,1] [2] [3] [4] [5,6]
+        plan.close()
+
+
+def test_the_library_refuses_a_stream_that_is_being_captured(cuda_device):
+    """Recorded into a graph the step would replay one step's bias correction for ever: FSADAM_EINVAL, nothing enqueued."""
+    from fairscale_amd import _cabi, fused_adam_hip
+
+    t = [torch.full((5000,), x, device=cuda_device) for x in (0.5, 0.0, 0.0, 0.01)]
+    flag = torch.zeros(1, device=cuda_device)
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(_cabi.FsAdamError, match="captured"):
+        with torch.cuda.graph(graph):
+            fused_adam_hip.adam(65536, None, [[x] for x in t], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)
+    torch.cuda.synchronize(cuda_device)
+    assert float(t[0][0]) == 0.5 and float(t[1].abs().max()) == 0.0
+    fused_adam_hip.adam(65536, None, [[x] for x in t], 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, flag, 1, 1, 1, 0.0)
+    torch.cuda.synchronize(cuda_device)
+    assert float(t[0][0]) != 0.5
 
 
 def _window_check(oracle, mode, before, after, grads, windows, kw, what):
