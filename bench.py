@@ -9,12 +9,23 @@ params and grads, fp32 m/v, grads scaled by 1024).  A "step" is one ``Adam.step(
 with everything resident in HBM.  Prints ONE JSON line; under "also": the same number of parameters
 stepped in the other three dtype combinations (MIXED_PRECISION = fp32 master + fp16 grads + fp16
 copy-out, 28 B/param; FULL_PRECISION 28; PURE_FP16 14), the pre-step gradient pass over the shard's
-fp16 gradients, and a list of 4096 ragged fp32 tensors (host time and device time per step).
+fp16 gradients, a list of 4096 ragged fp32 tensors (host time and device time per step; separately
+allocated, packed into flat buffers, with gradients that move every step), and the other benchmark
+configurations at their real sizes: "c1_..." (one fp32 tensor of 2^20, 10 steps with fresh gradients, on
+the host cores and on the GPU), "c2_..." (the 148-tensor GPT-2-small list, MIXED_PRECISION, gradients
+scaled by 65536) and "c5_..." (the 291-tensor Llama-7B list, PURE_FP16 with optimizer-state scaling,
+including one step whose gradients overflow the state: flag read-back, scale halved, state zeroed).
 
 "roofline" prices the dominant kernel against 8 TB/s of HBM: algorithmic bytes per launch (22 B per
 parameter in this mode: reads p16,g16,m32,v32, writes p16,m32,v32) over the kernel's average duration
-measured with HIP events on the launch stream.  "cpu_baseline" times the same math as in-place torch
-CPU ops on the host cores for a bounded sample.
+measured with HIP events on the launch stream over K back-to-back launches through the plan call of the
+C ABI ("kernel_ms_min/median/max": the spread over those launches, one event between every two;
+"ms_per_step" and "step_ms_median" are the same steps through ``Adam.step()``, which is what "value" counts).  "achieved" is therefore algorithmic bytes over event time; "traffic" is
+NOT measured by this run: it is the HBM byte count rocprofv3's counters gave for this workload at default
+options, read from the summary named in "traffic_source" (left out when options were changed).
+"cpu_baseline" times the same math as in-place torch CPU ops on the host cores for a bounded sample.
+
+    python bench.py --micro     the microbenchmarks the kernel's shape rests on (see run_micro)
 """
 from __future__ import annotations
 
@@ -46,6 +57,8 @@ def parse_args():
     ap.add_argument("--calib-copy-bytes", type=int, default=0,
                     help="first run the library's plain copy kernel over this many bytes three times (a dispatch of known "
                          "traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--micro", action="store_true", help="run the structure microbenchmarks instead (needs libfsadam_membench.so) and print a table")
+    ap.add_argument("--micro-numel", type=int, default=SHARD_NUMEL)
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (lds_throttle, merge_runs, align_heads, mid_tiles, ...)")
     return ap.parse_args()
 
@@ -66,21 +79,31 @@ def make_shard(torch, precision_name, numel, device):
     return p, scale
 
 
-def time_steps(torch, opt, scale, steps, warmup):
-    """W untimed steps, then K steps between synchronisations; wall time and HIP-event time (events sit
-    on torch's current stream, which is the stream the optimizer hands to the library)."""
-    for _ in range(warmup):
-        opt.step(scale=scale)
+def spread(values):
+    """min / median / max of a list of per-step times."""
+    ordered = sorted(values)
+    n = len(ordered)
+    median = ordered[n // 2] if n % 2 else 0.5 * (ordered[n // 2 - 1] + ordered[n // 2])
+    return {"min": ordered[0], "median": median, "max": ordered[-1]}
+
+
+def time_loop(torch, one_step, steps, warmup):
+    """W untimed steps, then K steps between synchronisations.  Returns (wall seconds until the device is idle,
+    host seconds until the last call returned, per-step device milliseconds).  The events sit on torch's current
+    stream, which is the stream the optimizer hands to the library; one event between every two steps."""
+    for i in range(warmup):
+        one_step(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        opt.step(scale=scale)
-    e1.record()
+    events[0].record()
+    for i in range(steps):
+        one_step(warmup + i)
+        events[i + 1].record()
+    host = time.perf_counter() - t0
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, e0.elapsed_time(e1) / 1e3
+    return wall, host, [events[i].elapsed_time(events[i + 1]) for i in range(steps)]
 
 
 def measure_gpu(torch, precision_name, numel, steps, warmup, device):
@@ -88,17 +111,35 @@ def measure_gpu(torch, precision_name, numel, steps, warmup, device):
 
     p, scale = make_shard(torch, precision_name, numel, device)
     opt = Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, precision=getattr(Precision, precision_name))
-    wall, dev_s = time_steps(torch, opt, scale, steps, warmup)
-    plan = next(iter(opt._plans.values())).info()
+    wall, _, per_step = time_loop(torch, lambda i: opt.step(scale=scale), steps, warmup)
+    plan_obj = next(iter(opt._plans.values()))
+    plan = plan_obj.info()
     assert torch.isfinite(p.detach()[:4096].float()).all()
     bpp = BYTES_PER_PARAM[precision_name]
-    kernel_s = dev_s / steps  # one launch per step: plan["n_launches"] == 1
+    sp = spread(per_step)
+    # The kernel on its own: the same launches through the plan call of the C ABI, back to back without the host in
+    # between.  In PURE_FP16 Adam.step() reads the overflow flag back after every launch (as the reference does,
+    # adam.py:278), which leaves the GPU idle until the host has seen the flag and queued the next step; the other
+    # modes never wait, and the two figures agree.
+    flag = opt._flags.get(device)
+    done = opt.state[p]["step"]
+    group = opt.param_groups[0]
+
+    def launch_only(i):
+        plan_obj.step_rows(False, group["lr"], group["betas"][0], group["betas"][1], group["eps"], scale, opt._optim_scale, flag,
+                           done + 1 + i, opt.eps_mode, 1, group["weight_decay"])
+
+    _, _, raw = time_loop(torch, launch_only, steps, 2)
+    kernel_ms = sum(raw) / steps  # one launch per step: plan["n_launches"] == 1
+    raw_sp = spread(raw)
     out = {
         "params_per_s": numel * steps / wall,
         "ms_per_step": wall / steps * 1e3,
-        "kernel_ms": kernel_s * 1e3,
+        "step_ms_min": sp["min"], "step_ms_median": sp["median"], "step_ms_max": sp["max"],
+        "kernel_ms": kernel_ms,
+        "kernel_ms_min": raw_sp["min"], "kernel_ms_median": raw_sp["median"], "kernel_ms_max": raw_sp["max"],
         "bytes_per_param": bpp,
-        "achieved_gbs": numel * bpp / kernel_s / 1e9,
+        "achieved_gbs": numel * bpp / kernel_ms / 1e6,
         "plan": {k: plan[k] for k in ("n_launches", "grid", "block", "tile_elems", "n_descriptors", "lds_throttle", "n_vector_tensors")},
     }
     del opt, p
@@ -142,24 +183,15 @@ def measure_ragged(torch, steps, warmup, device, count=4096, seed=3000, packed=F
                 p.grad = g
         opt.step()
 
-    for i in range(warmup):
-        one_step(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        one_step(warmup + i)
-    e1.record()
-    host = time.perf_counter() - t0
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall, host, per_step = time_loop(torch, one_step, steps, warmup)
     total = sum(sizes)
     plan = next(iter(opt._plans.values())).info()
-    out = {"tensors": count, "numel": total, "host_ms_per_step": host / steps * 1e3, "device_ms_per_step": e0.elapsed_time(e1) / steps,
+    sp = spread(per_step)
+    out = {"tensors": count, "numel": total, "host_ms_per_step": host / steps * 1e3, "device_ms_per_step": sum(per_step) / steps,
+           "device_ms_min": sp["min"], "device_ms_median": sp["median"], "device_ms_max": sp["max"],
            "ms_per_step": wall / steps * 1e3, "params_per_s": total * steps / wall, "bytes_per_param": 28,
            "achieved_gbs": total * 28 * steps / wall / 1e9, "frac_of_hbm_peak": total * 28 * steps / wall / 1e9 / HBM_PEAK_GBS,
-           "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "uploads": plan["uploads"],
+           "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "n_runs": plan["n_runs"], "uploads": plan["uploads"],
            "list_walk": "c++" if _rows.native is not None else "python"}
     del opt, params, sets
     torch.cuda.empty_cache()
@@ -187,6 +219,152 @@ def measure_grad_pass(torch, numel, steps, warmup, device):
         ms = e0.elapsed_time(e1) / steps
         out[name] = {"ms": ms, "bytes_per_param": bpp, "achieved_gbs": numel * bpp / ms / 1e6, "frac_of_hbm_peak": numel * bpp / ms / 1e6 / HBM_PEAK_GBS}
     del g
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_c1(torch, device):
+    """Benchmark configuration 1 exactly, on the host cores and on the GPU: ONE fp32 tensor of 2^20 parameters
+    ~N(0, 0.02) (seed 1000), m = v = 0, lr 1e-3, betas (0.9, 0.999), eps 1e-8 outside the square root, no weight decay,
+    10 steps with fresh gradients ~N(0, 1e-3) (seed 1000 + step), all drawn on the CPU in float32.  The CPU leg is the
+    same math as in-place torch CPU ops on all host cores; the GPU leg is ``Adam.step()`` (the working set, 16 MiB, sits
+    in the caches: its rate says nothing about HBM).  The two results are compared (they differ by the order of
+    torch's CPU loops, so to a tolerance)."""
+    from fairscale_amd.optim import Adam, Precision
+    from oracle import adam_oracle as O
+    from oracle.adam_torch_cpu import step_torch_cpu
+
+    n, steps = 1 << 20, 10
+    p0 = torch.randn(n, generator=torch.Generator().manual_seed(1000)) * 0.02
+    grads = [torch.randn(n, generator=torch.Generator().manual_seed(1000 + step)) * 1e-3 for step in range(1, steps + 1)]
+    kw = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    times = []
+    for rep in range(3):  # the third repetition is the one reported (threads and pages warm)
+        p, m, v = p0.clone(), torch.zeros(n), torch.zeros(n)
+        t0 = time.perf_counter()
+        for step, g in enumerate(grads, 1):
+            step_torch_cpu(O.FULL_PRECISION, p, m, v, g, None, step=step, **kw)
+        times.append(time.perf_counter() - t0)
+    cpu_s = times[-1]
+    q = p0.to(device).requires_grad_()
+    dev_grads = [g.to(device) for g in grads]
+    opt = Adam([q], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, precision=Precision.FULL_PRECISION)
+    torch.cuda.synchronize()
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    events[0].record()
+    for i, g in enumerate(dev_grads):
+        q.grad = g  # another tensor every step, as after zero_grad(set_to_none=True)
+        opt.step()
+        events[i + 1].record()
+    torch.cuda.synchronize()
+    gpu_s = time.perf_counter() - t0
+    per_step = [events[i].elapsed_time(events[i + 1]) for i in range(steps)]
+    diff = (q.detach().cpu() - p).abs().max().item() / p.abs().max().item()
+    assert diff < 1e-6, f"C1: GPU and CPU results differ by {diff}"
+    sp = spread(per_step[1:])  # the first step creates the state and the plan
+    return {"numel": n, "steps": steps, "cpu": {"params_per_s": n * steps / cpu_s, "ms_per_step": cpu_s / steps * 1e3, "cores": int(torch.get_num_threads()),
+                                                 "kind": "port (oracle/adam_torch_cpu.py, in-place torch CPU ops)"},
+            "gpu": {"params_per_s": n * steps / gpu_s, "ms_per_step": gpu_s / steps * 1e3, "device_ms_min": sp["min"], "device_ms_median": sp["median"],
+                    "device_ms_max": sp["max"], "note": "10 steps from a cold optimizer, wall time; 16 MiB working set, cache-resident"},
+            "max_abs_diff_over_max_abs": diff}
+
+
+def measure_c2(torch, steps, warmup, device):
+    """Benchmark configuration 2: the GPT-2-small list (148 tensors, 124 439 808 parameters) in MIXED_PRECISION -- fp32
+    master copies, m and v; fp16 gradients pre-scaled by 65536 and the same number passed as ``scale``; fp16 parameters
+    written in the same pass -- through ``Adam.step()``.  28 bytes per parameter."""
+    from fairscale_amd.optim import Adam, Precision
+
+    shapes = [(50257, 768), (1024, 768)]
+    for _ in range(12):
+        shapes += [(768,), (768,), (768, 2304), (2304,), (768, 768), (768,), (768,), (768,), (768, 3072), (3072,), (3072, 768), (768,)]
+    shapes += [(768,), (768,)]
+    gen = torch.Generator(device=device).manual_seed(2000)
+    params = [torch.empty(sh, device=device, dtype=torch.float16).normal_(0, 0.02, generator=gen).requires_grad_() for sh in shapes]
+    for p in params:
+        p.grad = torch.empty_like(p).normal_(0, 1e-3 * 65536, generator=gen)
+    opt = Adam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, precision=Precision.MIXED_PRECISION)
+    wall, host, per_step = time_loop(torch, lambda i: opt.step(scale=65536.0), steps, warmup)
+    total = sum(p.numel() for p in params)
+    assert len(params) == 148 and total == 124_439_808
+    plan = next(iter(opt._plans.values())).info()
+    sp = spread(per_step)
+    assert all(torch.isfinite(p.detach()[..., :64].float()).all() for p in params[:3])
+    out = {"tensors": 148, "numel": total, "ms_per_step": wall / steps * 1e3, "host_ms_per_step": host / steps * 1e3,
+           "device_ms_min": sp["min"], "device_ms_median": sp["median"], "device_ms_max": sp["max"], "params_per_s": total * steps / wall,
+           "bytes_per_param": 28, "achieved_gbs": total * 28 * steps / wall / 1e9, "frac_of_hbm_peak": total * 28 * steps / wall / 1e9 / HBM_PEAK_GBS,
+           "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "n_runs": plan["n_runs"], "grad_scale": 65536.0,
+           "note": "3.5 GB working set"}
+    del opt, params
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_c5(torch, steps, warmup, device):
+    """Benchmark configuration 5: the Llama-7B list (291 tensors, 6 738 415 616 parameters; 32 layers, hidden 4096, FFN
+    11008, vocabulary 32000) in PURE_FP16 -- fp16 parameters, gradients, m and v, optimizer-state scale 2^16 -- through
+    ``Adam.step()``, which reads the overflow flag back every step as the reference does.  After the clean steps one step
+    runs with 1 gradient element in 10^6 set to 6e4: the stored second moment overflows, the flag comes back raised, the
+    scale is halved and all of m and v is zeroed (27 GB); that step is timed on its own and its effects are asserted,
+    then one more clean step runs at the halved scale.  14 bytes per parameter."""
+    from fairscale_amd.optim import Adam, Precision
+
+    h, f, vocab = 4096, 11008, 32000
+    shapes = [(vocab, h)]
+    for _ in range(32):
+        shapes += [(h, h)] * 4 + [(f, h), (h, f), (f, h), (h,), (h,)]
+    shapes += [(h,), (vocab, h)]
+    total = sum(a * (b[0] if b else 1) for a, *b in shapes)
+    assert len(shapes) == 291 and total == 6_738_415_616
+    free, _ = torch.cuda.mem_get_info(device)
+    if free < total * 8 + (8 << 30):
+        return {"skipped": f"needs {(total * 8 >> 30) + 8} GiB of device memory, {free >> 30} GiB free"}
+    gen = torch.Generator(device=device).manual_seed(5000)
+    params = [torch.empty(sh, device=device, dtype=torch.float16).normal_(0, 0.02, generator=gen).requires_grad_() for sh in shapes]
+    for p in params:
+        p.grad = torch.empty_like(p).normal_(0, 1e-3, generator=gen)
+    opt = Adam(params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, precision=Precision.PURE_FP16)
+    wall, host, per_step = time_loop(torch, lambda i: opt.step(), steps, warmup)
+    assert opt._optim_scale == 65536.0 and opt._steps_since_optim_scale_change == steps + warmup
+    sp = spread(per_step)
+    # the overflow step
+    cpu_gen = torch.Generator().manual_seed(5002)
+    saved = []
+    for p in params:
+        k = p.numel() // 1_000_000
+        if k:
+            idx = torch.randint(0, p.numel(), (k,), generator=cpu_gen).to(device)
+            flat = p.grad.view(-1)
+            saved.append((flat, idx, flat[idx].clone()))
+            flat[idx] = 6e4
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    opt.step()
+    torch.cuda.synchronize()
+    overflow_ms = (time.perf_counter() - t0) * 1e3
+    assert opt._optim_scale == 32768.0 and opt._steps_since_optim_scale_change == 0, "the overflow was not acted upon"
+    zeroed = all(not bool(opt.state[p][key].any()) for p in params for key in ("exp_avg", "exp_avg_sq"))
+    assert zeroed, "m and v were not zeroed after the overflow"
+    for flat, idx, old in saved:
+        flat[idx] = old
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    opt.step()
+    torch.cuda.synchronize()
+    after_ms = (time.perf_counter() - t0) * 1e3
+    assert opt._optim_scale == 32768.0 and opt._steps_since_optim_scale_change == 1
+    plan = next(iter(opt._plans.values())).info()
+    out = {"tensors": 291, "numel": total, "ms_per_step": wall / steps * 1e3, "host_ms_per_step": host / steps * 1e3,
+           "device_ms_min": sp["min"], "device_ms_median": sp["median"], "device_ms_max": sp["max"], "params_per_s": total * steps / wall,
+           "bytes_per_param": 14, "achieved_gbs": total * 14 * steps / wall / 1e9, "frac_of_hbm_peak": total * 14 * steps / wall / 1e9 / HBM_PEAK_GBS,
+           "n_launches": plan["n_launches"], "n_descriptors": plan["n_descriptors"], "n_runs": plan["n_runs"],
+           "overflow_step": {"ms": overflow_ms, "injected": "1 gradient element in 10^6 set to 6e4", "optim_scale_before": 65536.0,
+                             "optim_scale_after": opt._optim_scale, "state_zeroed": zeroed,
+                             "note": "step + blocking flag read-back + scale halved + m, v of all 291 tensors zeroed in place (27 GB written)"},
+           "clean_step_after_backoff_ms": after_ms,
+           "note": "every step includes the blocking read-back of the overflow flag, as in the reference (adam.py:278)"}
+    del opt, params, saved
     torch.cuda.empty_cache()
     return out
 
@@ -239,6 +417,88 @@ def load_traffic(workload_key):
     return int(found.group(1)) if found else None
 
 
+def run_micro(torch, args, device):
+    """The measurements the kernel's shape rests on, from kernels the tree builds (fairscale_amd/csrc/membench.hip):
+    one-shot tiles against a grid-stride loop, residency (LDS ballast) sweep, temporal against non-temporal accesses,
+    the descriptor read with one scalar load against a descriptor staged in LDS, and the ceilings of this part for reads
+    only, writes only and the step's mix.  Prints one line per variant and one JSON line at the end."""
+    import ctypes
+
+    path = os.path.join(REPO, "fairscale_amd", "csrc", "libfsadam_membench.so")
+    if not os.path.exists(path):
+        print(f"{path} is missing: build it with `python -m fairscale_amd.csrc.build`", file=sys.stderr)
+        sys.exit(1)
+    L = ctypes.CDLL(path)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    L.fsadam_membench_launch.restype = i32
+    L.fsadam_membench_launch.argtypes = [i32, vp, vp, vp, vp, i64, i32, i32, vp, vp, vp]
+    L.fsadam_membench_table_bytes.restype = i64
+    L.fsadam_membench_table_bytes.argtypes = [i64]
+    n = args.micro_numel // 4 * 4
+    bufs = [torch.zeros(n, device=device, dtype=torch.float32) for _ in range(4)]
+    table = torch.zeros(L.fsadam_membench_table_bytes(n), device=device, dtype=torch.uint8)
+    sink = torch.zeros(1, device=device)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch(kind, lds=0, param=0):
+        rc = L.fsadam_membench_launch(kind, *(b.data_ptr() for b in bufs), n, lds, param, table.data_ptr(), sink.data_ptr(), stream)
+        assert rc == 0, f"membench variant {kind} returned {rc}"
+
+    launch(-1)
+    results = []
+
+    def measure(name, kind, bytes_per_elt, lds=0, param=0, iters=10):
+        for _ in range(3):
+            launch(kind, lds, param)
+        torch.cuda.synchronize()
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1)]
+        events[0].record()
+        for i in range(iters):
+            launch(kind, lds, param)
+            events[i + 1].record()
+        torch.cuda.synchronize()
+        times = [events[i].elapsed_time(events[i + 1]) for i in range(iters)]
+        sp = spread(times)
+        gbs = n * bytes_per_elt / sp["median"] / 1e6
+        results.append({"variant": name, "kind": kind, "lds_bytes": lds, "param": param, "bytes_per_element": bytes_per_elt,
+                        "ms_median": sp["median"], "ms_min": sp["min"], "gbs_at_median": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
+        print(f"{name:<78s} {sp['median']:8.3f} ms  {gbs:7.0f} GB/s  {gbs / HBM_PEAK_GBS * 100:5.1f} %", flush=True)
+
+    print(f"# {n} elements per stream; GB/s of algorithmic bytes at the median of 10 launches; peak {HBM_PEAK_GBS:.0f} GB/s")
+    print("# fp32 shape: p, m, v, g read, p, m, v written (28 B/element)")
+    for wg in (4, 8, 16):
+        measure(f"grid-stride loop, 256 threads, {wg} workgroups per CU, non-temporal", 1, 28, param=wg)
+    measure("one-shot tiles (one wave64 each), full residency, non-temporal", 0, 28)
+    measure("one-shot tiles, full residency, plain (temporal) loads and stores", 2, 28)
+    for lds in (5120, 8192, 10240, 12288, 13312, 16384, 20480, 26624, 32768, 65536):
+        measure(f"one-shot tiles, LDS ballast {lds:5d} B (at most {163840 // lds:2d} waves per CU), non-temporal", 0, 28, lds=lds)
+    measure("one-shot tiles, ballast 16384 B, plain (temporal) loads and stores", 2, 28, lds=16384)
+    measure("table of descriptors, ONE scalar load per wave, ballast 16384 B", 4, 28, lds=16384)
+    measure("table of descriptors staged in LDS + barrier, ballast 16384 B (incl. the 64 B staged)", 3, 28, lds=16384 - 64)
+    measure("table of descriptors staged in LDS + barrier, no ballast", 3, 28)
+    measure("reads only, four fp32 streams (16 B/element), ballast 16384 B", 5, 16, lds=16384)
+    measure("writes only, three fp32 streams (12 B/element), ballast 16384 B", 6, 12, lds=16384)
+    print("# the write side on its own (fp32 streams)")
+    for lds in (0, 8192, 12288, 20480, 32768):
+        measure(f"writes only, three streams, ballast {lds:5d} B", 6, 12, lds=lds)
+    measure("writes only, three streams, plain (temporal) stores, ballast 16384 B", 11, 12, lds=16384)
+    measure("writes only, three streams, 4 KiB per wave and stream, ballast 32768 B", 12, 12, lds=32768)
+    measure("writes only, ONE stream (a fill), ballast 16384 B", 10, 4, lds=16384)
+    measure("writes only, ONE stream (a fill), no ballast", 10, 4)
+    for lds in (32768, 53248, 81920):
+        measure(f"28 B shape, four vectors per lane: 16 loads, then 12 stores, ballast {lds:5d} B", 13, 28, lds=lds)
+    print("# MEMORY_EFFICIENT shape: p, g fp16 and m, v fp32 read (12 B/element), p, m, v written (10 B/element)")
+    measure("reads only (12 B/element), ballast 12288 B", 7, 12, lds=12288)
+    measure("writes only (10 B/element), ballast 12288 B", 8, 10, lds=12288)
+    measure("reads and writes (22 B/element), ballast 12288 B", 9, 22, lds=12288)
+    by = {r["variant"]: r for r in results}
+    r_gbs = by["reads only (12 B/element), ballast 12288 B"]["gbs_at_median"]
+    w_gbs = by["writes only (10 B/element), ballast 12288 B"]["gbs_at_median"]
+    serial = 22.0 / (12.0 / r_gbs + 10.0 / w_gbs)
+    print(f"# 12 B read at {r_gbs:.0f} GB/s + 10 B written at {w_gbs:.0f} GB/s, one after the other: {serial:.0f} GB/s = {serial / HBM_PEAK_GBS * 100:.1f} % of peak")
+    print(json.dumps({"micro": results, "numel": n, "memeff_mix_ceiling_gbs": serial}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -258,6 +518,9 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.micro:
+        run_micro(torch, args, device)
+        return
     if args.calib_copy_bytes > 0:
         n = args.calib_copy_bytes // 16 * 16
         src = torch.zeros(n, dtype=torch.uint8, device=device)
@@ -276,17 +539,27 @@ def main():
             if mode == args.mode:
                 continue
             r = measure_gpu(torch, mode, args.numel, args.steps, args.warmup, device)
-            also[mode] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
-                          "bytes_per_param": r["bytes_per_param"], "achieved_gbs": r["achieved_gbs"],
-                          "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS}
+            also[mode] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "step_ms_median": r["step_ms_median"],
+                          "kernel_ms": r["kernel_ms"], "kernel_ms_min": r["kernel_ms_min"], "kernel_ms_median": r["kernel_ms_median"],
+                          "kernel_ms_max": r["kernel_ms_max"], "bytes_per_param": r["bytes_per_param"], "achieved_gbs": r["achieved_gbs"],
+                          "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS,
+                          "frac_of_hbm_peak_through_adam_step": args.numel * r["bytes_per_param"] / r["ms_per_step"] / 1e6 / HBM_PEAK_GBS}
     if not args.no_also:
         also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
         also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device)
         also["ragged_4096_packed_views_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device, packed=True)
         also["ragged_4096_moving_gradients_FULL_PRECISION"] = measure_ragged(torch, args.steps, args.warmup, device, moving=True)
+        also["c2_gpt2_small_148_tensors_MIXED_PRECISION"] = measure_c2(torch, args.steps, args.warmup, device)
+        also["c5_llama7b_291_tensors_PURE_FP16"] = measure_c5(torch, min(args.steps, 10), min(args.warmup, 3), device)
+        if not args.no_cpu:
+            also["c1_flat_2pow20_FULL_PRECISION_10_steps"] = measure_c1(torch, device)
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"
+    # the committed counter summary speaks for default options only
+    traffic = load_traffic(workload) if not args.opt else None
+    traffic_source = (f"profiles/{TRAFFIC_SUMMARIES[workload]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload at default options; "
+                      "not measured by this run)") if traffic is not None else None
     line = {
         "metric": "params updated/sec + HBM GB/s (% of peak), 1.6B-param shard, mixed precision",
         "value": main_res["params_per_s"],
@@ -306,8 +579,12 @@ def main():
                    "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
                    "options": {k: _cabi.get_option(k) for k in ("lds_throttle", "merge_runs", "align_heads", "mid_tiles")}},
         "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": load_traffic(workload),
-                     "kernel": "fsadam_tiles", "kernel_ms": main_res["kernel_ms"], "bytes_per_param": main_res["bytes_per_param"]},
+                     "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "fsadam_tiles", "kernel_ms": main_res["kernel_ms"], "step_ms_median": main_res["step_ms_median"],
+                     "kernel_ms_min": main_res["kernel_ms_min"],
+                     "kernel_ms_median": main_res["kernel_ms_median"], "kernel_ms_max": main_res["kernel_ms_max"],
+                     "frac_at_median": args.numel * main_res["bytes_per_param"] / main_res["kernel_ms_median"] / 1e6 / HBM_PEAK_GBS,
+                     "bytes_per_param": main_res["bytes_per_param"]},
         "cpu_baseline": cpu,
         "also": also,
     }

@@ -47,6 +47,24 @@ def build_library(verbose: bool = False) -> str:
     return LIBRARY
 
 
+MEMBENCH_SOURCE = os.path.join(HERE, "membench.hip")
+MEMBENCH_LIBRARY = os.path.join(HERE, "libfsadam_membench.so")
+
+
+def build_membench(verbose: bool = False) -> str:
+    """The microbenchmark kernels of ``bench.py --micro`` (a library of their own: nothing in the product loads it)."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", MEMBENCH_LIBRARY + ".tmp", MEMBENCH_SOURCE]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    noise = "is not a recognized feature for this target"
+    log = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
+    os.replace(MEMBENCH_LIBRARY + ".tmp", MEMBENCH_LIBRARY)
+    if verbose and log.strip():
+        print(log, file=sys.stderr)
+    return MEMBENCH_LIBRARY
+
+
 ROWS_SOURCE = os.path.join(HERE, "tensor_rows.cpp")
 
 
@@ -86,4 +104,5 @@ def build_rows_module(verbose: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_membench(verbose=True))
     print(build_rows_module(verbose=True))

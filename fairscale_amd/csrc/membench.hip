@@ -1,0 +1,294 @@
+// Microbenchmarks of the memory-access structures the Adam kernels were chosen among (MI355X, gfx950).
+// Not part of the product: built into libfsadam_membench.so, driven by `bench.py --micro`, which times
+// the launches with HIP events and prints a table.  Every kernel moves the streams of an Adam step with
+// trivial arithmetic (two multiply-adds per element), so that what is measured is the memory system:
+//   * four fp32 streams p, m, v, g of `n` elements, read (all four) and written back (p, m, v): 28 bytes
+//     per element, the FULL_PRECISION shape; or
+//   * the MEMORY_EFFICIENT shape: p, g fp16 (2 bytes), m, v fp32: 12 bytes read, 10 written per element.
+// One entry point launches one variant once on the caller's stream; nothing is allocated here.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#define FS_GLOBAL __attribute__((address_space(1)))
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+template <bool NT, typename T>
+__device__ __forceinline__ T ld(FS_GLOBAL const T* p) {
+    return NT ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void st(FS_GLOBAL T* p, T v) {
+    if (NT) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+
+// the stand-in for the update: enough arithmetic to keep every loaded value alive, nothing more
+__device__ __forceinline__ void fake_update(f4& p, f4& m, f4& v, f4 g) {
+    m = m * 0.9f + g * 0.1f;
+    v = v * 0.999f + g * g * 0.001f;
+    p = p - m * 0.001f;
+}
+
+// ---- variant 0/2: one-shot tiles.  One workgroup = one wave64 = 64 quads per stream, then it exits.
+template <bool NT>
+__global__ __launch_bounds__(64) void mb_oneshot(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + i;
+    f4 a = ld<NT>((FS_GLOBAL const f4*)p), b = ld<NT>((FS_GLOBAL const f4*)m), c = ld<NT>((FS_GLOBAL const f4*)v),
+       d = ld<NT>((FS_GLOBAL const f4*)g_ + i);
+    fake_update(a, b, c, d);
+    st<NT>(m, b);
+    st<NT>(v, c);
+    st<NT>(p, a);
+}
+
+// ---- variant 1: persistent workgroups of 256 threads in a grid-stride loop (grid = CUs x workgroups per CU).
+__global__ __launch_bounds__(256) void mb_gridstride(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq) {
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_;
+    FS_GLOBAL const f4* g = (FS_GLOBAL const f4*)g_;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nq; i += (int64_t)gridDim.x * 256) {
+        f4 a = ld<true>((FS_GLOBAL const f4*)p + i), b = ld<true>((FS_GLOBAL const f4*)m + i), c = ld<true>((FS_GLOBAL const f4*)v + i),
+           d = ld<true>(g + i);
+        fake_update(a, b, c, d);
+        st<true>(m + i, b);
+        st<true>(v + i, c);
+        st<true>(p + i, a);
+    }
+}
+
+// ---- variants 3/4: the pointers come from a table of 64-byte descriptors in device memory (one per chunk of
+// `tiles_per_desc` tiles), as in the multi-tensor step.
+struct alignas(64) MbDesc {
+    f4* p;
+    f4* m;
+    f4* v;
+    const f4* g;
+    uint64_t nq;  // quads in this chunk
+    uint64_t pad[3];
+};
+
+// 4: one scalar load of the whole descriptor (uniform address, constant address space) per wave -- the product's way
+__global__ __launch_bounds__(64) void mb_table_scalar(const MbDesc* table, uint32_t log2_tiles) {
+    const uint32_t chunk = blockIdx.x >> log2_tiles, tile = blockIdx.x & ((1u << log2_tiles) - 1u);
+    typedef uint32_t words_t __attribute__((ext_vector_type(16)));
+    const words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) words_t*>((const __attribute__((address_space(4))) MbDesc*)table + chunk);
+    const MbDesc d = __builtin_bit_cast(MbDesc, raw);
+    const uint64_t i = (uint64_t)tile * 64 + threadIdx.x;
+    if (i >= d.nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)d.p + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)d.m + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)d.v + i;
+    f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+       e = ld<true>((FS_GLOBAL const f4*)d.g + i);
+    fake_update(a, b, c, e);
+    st<true>(m, b);
+    st<true>(v, c);
+    st<true>(p, a);
+}
+
+// 3: the descriptor is staged in LDS by the workgroup's first lanes, the workgroup synchronises, and every lane reads
+// the pointers from LDS -- the structure of a launcher whose metadata lives in shared memory
+__global__ __launch_bounds__(64) void mb_table_lds(const MbDesc* table, uint32_t log2_tiles) {
+    __shared__ MbDesc staged;
+    const uint32_t chunk = blockIdx.x >> log2_tiles, tile = blockIdx.x & ((1u << log2_tiles) - 1u);
+    if (threadIdx.x < 16) reinterpret_cast<uint32_t*>(&staged)[threadIdx.x] = reinterpret_cast<const uint32_t*>(table + chunk)[threadIdx.x];
+    __syncthreads();
+    const uint64_t i = (uint64_t)tile * 64 + threadIdx.x;
+    if (i >= staged.nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)staged.p + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)staged.m + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)staged.v + i;
+    f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+       e = ld<true>((FS_GLOBAL const f4*)staged.g + i);
+    fake_update(a, b, c, e);
+    st<true>(m, b);
+    st<true>(v, c);
+    st<true>(p, a);
+}
+
+// ---- variants 5/6: the fp32 streams one direction at a time (one-shot tiles).
+__global__ __launch_bounds__(64) void mb_read4(const f4* p_, const f4* m_, const f4* v_, const f4* g_, int64_t nq, float* sink) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 s = ld<true>((FS_GLOBAL const f4*)p_ + i) + ld<true>((FS_GLOBAL const f4*)m_ + i) + ld<true>((FS_GLOBAL const f4*)v_ + i) +
+                 ld<true>((FS_GLOBAL const f4*)g_ + i);
+    if (s[0] + s[1] + s[2] + s[3] == 12345.678f) *sink = 1.0f;  // never true for the zero-filled buffers: keeps the loads
+}
+__global__ __launch_bounds__(64) void mb_write3(f4* p_, f4* m_, f4* v_, int64_t nq) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    st<true>((FS_GLOBAL f4*)m_ + i, val);
+    st<true>((FS_GLOBAL f4*)v_ + i, val);
+    st<true>((FS_GLOBAL f4*)p_ + i, val);
+}
+
+// ---- variants 7/8/9: the MEMORY_EFFICIENT shape (4 elements per lane: 8 bytes of the fp16 streams, 16 of the fp32 ones):
+// reads only (12 B/elt), writes only (10 B/elt), both (22 B/elt).  `n4` = groups of 4 elements.
+__global__ __launch_bounds__(64) void mb_memeff_read(const f2* p_, const f4* m_, const f4* v_, const f2* g_, int64_t n4, float* sink) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    const f2 a = ld<true>((FS_GLOBAL const f2*)p_ + i), d = ld<true>((FS_GLOBAL const f2*)g_ + i);
+    const f4 s = ld<true>((FS_GLOBAL const f4*)m_ + i) + ld<true>((FS_GLOBAL const f4*)v_ + i);
+    if (s[0] + s[1] + s[2] + s[3] + a[0] + a[1] + d[0] + d[1] == 12345.678f) *sink = 1.0f;
+}
+__global__ __launch_bounds__(64) void mb_memeff_write(f2* p_, f4* m_, f4* v_, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f2 half = {0.f, 0.f};
+    st<true>((FS_GLOBAL f4*)m_ + i, val);
+    st<true>((FS_GLOBAL f4*)v_ + i, val);
+    st<true>((FS_GLOBAL f2*)p_ + i, half);
+}
+__global__ __launch_bounds__(64) void mb_memeff_both(f2* p_, f4* m_, f4* v_, const f2* g_, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    f2 a = ld<true>((FS_GLOBAL const f2*)p_ + i);
+    const f2 d = ld<true>((FS_GLOBAL const f2*)g_ + i);
+    f4 b = ld<true>((FS_GLOBAL const f4*)m_ + i), c = ld<true>((FS_GLOBAL const f4*)v_ + i);
+    const f4 g = {d[0], d[1], d[0], d[1]};
+    b = b * 0.9f + g * 0.1f;
+    c = c * 0.999f + g * g * 0.001f;
+    a[0] -= b[0] * 0.001f;
+    a[1] -= b[1] * 0.001f;
+    st<true>((FS_GLOBAL f4*)m_ + i, b);
+    st<true>((FS_GLOBAL f4*)v_ + i, c);
+    st<true>((FS_GLOBAL f2*)p_ + i, a);
+}
+
+// ---- variants 10-13: what else could be done about the write side.
+// 10: ONE stream written (a fill); 11: three streams with plain (temporal) stores; 12: three streams, every wave
+// writes four consecutive vectors per stream (4 KiB bursts); 13: the 28-byte shape with four vectors per lane and
+// stream: all sixteen loads first, then all twelve stores (longer same-direction bursts per wave).
+__global__ __launch_bounds__(64) void mb_write1(f4* p_, int64_t nq) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    st<true>((FS_GLOBAL f4*)p_ + i, val);
+}
+__global__ __launch_bounds__(64) void mb_write3_temporal(f4* p_, f4* m_, f4* v_, int64_t nq) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    st<false>((FS_GLOBAL f4*)m_ + i, val);
+    st<false>((FS_GLOBAL f4*)v_ + i, val);
+    st<false>((FS_GLOBAL f4*)p_ + i, val);
+}
+__global__ __launch_bounds__(64) void mb_write3_bursts(f4* p_, f4* m_, f4* v_, int64_t nq) {
+    const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) if (base + k * 64 < nq) st<true>((FS_GLOBAL f4*)m_ + base + k * 64, val);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) if (base + k * 64 < nq) st<true>((FS_GLOBAL f4*)v_ + base + k * 64, val);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) if (base + k * 64 < nq) st<true>((FS_GLOBAL f4*)p_ + base + k * 64, val);
+}
+__global__ __launch_bounds__(64) void mb_oneshot_x4(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq) {
+    const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (base + 192 >= nq) return;  // the ragged end is left out: a handful of quads in 4e8
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + base;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + base;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + base;
+    FS_GLOBAL const f4* g = (FS_GLOBAL const f4*)g_ + base;
+    f4 a[4], b[4], c[4], d[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        a[k] = ld<true>((FS_GLOBAL const f4*)p + k * 64); b[k] = ld<true>((FS_GLOBAL const f4*)m + k * 64);
+        c[k] = ld<true>((FS_GLOBAL const f4*)v + k * 64); d[k] = ld<true>(g + k * 64);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fake_update(a[k], b[k], c[k], d[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(m + k * 64, b[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(v + k * 64, c[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(p + k * 64, a[k]);
+}
+
+// fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
+__global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
+    const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= n_desc) return;
+    const uint64_t first = (uint64_t)k * chunk_q;
+    MbDesc d = {};
+    d.p = p + first; d.m = m + first; d.v = v + first; d.g = g + first;
+    d.nq = nq - first < chunk_q ? nq - first : chunk_q;
+    table[k] = d;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Bytes the caller must provide for the descriptor table of variants 3 and 4 (chunks of 2^16 quads).
+int64_t fsadam_membench_table_bytes(int64_t numel) {
+    const int64_t nq = numel / 4, chunk_q = 1 << 16;
+    return ((nq + chunk_q - 1) / chunk_q) * (int64_t)sizeof(MbDesc);
+}
+
+// Launches variant `kind` once over `numel` elements (a multiple of 4) on `stream`.  p, m, v, g: device buffers of
+// numel floats (the MEMORY_EFFICIENT variants use the first half of p and g as fp16).  lds_bytes: untouched LDS given to
+// every workgroup (caps residency).  param: variant 1: workgroups per compute unit.  table: device memory of
+// fsadam_membench_table_bytes(numel) bytes for variants 3, 4 and -1 (-1 fills it; do that once before them).
+// Returns 0, or -1 for an unknown kind / bad argument, -2 for a launch error.
+int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t numel, int lds_bytes, int param, void* table, void* sink,
+                           void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (numel <= 0 || (numel & 3) || !p || !m || !v || !g) return -1;
+    const int64_t nq = numel / 4;
+    const int64_t grid64 = (nq + 63) / 64;
+    if (grid64 > 0x7ffffff0) return -1;
+    f4 *P = (f4*)p, *M = (f4*)m, *V = (f4*)v;
+    const f4* G = (const f4*)g;
+    const size_t lds = (size_t)lds_bytes;
+    const int64_t chunk_q = 1 << 16;
+    const uint32_t n_desc = (uint32_t)((nq + chunk_q - 1) / chunk_q);
+    switch (kind) {
+        case -1:
+            if (!table) return -1;
+            hipLaunchKernelGGL(mb_fill_table, dim3((n_desc + 255) / 256), dim3(256), 0, stream, (MbDesc*)table, P, M, V, G, (uint64_t)nq, (uint64_t)chunk_q, n_desc);
+            break;
+        case 0: hipLaunchKernelGGL(mb_oneshot<true>, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq); break;
+        case 1: {
+            int dev = 0, cus = 256;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -2;
+            hipLaunchKernelGGL(mb_gridstride, dim3((uint32_t)(cus * (param > 0 ? param : 8))), dim3(256), lds, stream, P, M, V, G, nq);
+            break;
+        }
+        case 2: hipLaunchKernelGGL(mb_oneshot<false>, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq); break;
+        case 3:
+        case 4: {
+            if (!table) return -1;
+            const uint32_t log2_tiles = 10;  // 2^16 quads per descriptor / 64 quads per tile
+            const uint32_t grid = n_desc << log2_tiles;
+            if (kind == 3) hipLaunchKernelGGL(mb_table_lds, dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            else hipLaunchKernelGGL(mb_table_scalar, dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            break;
+        }
+        case 5: hipLaunchKernelGGL(mb_read4, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq, (float*)sink); break;
+        case 6: hipLaunchKernelGGL(mb_write3, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq); break;
+        case 7: hipLaunchKernelGGL(mb_memeff_read, dim3((uint32_t)grid64), dim3(64), lds, stream, (const f2*)p, M, V, (const f2*)g, nq, (float*)sink); break;
+        case 8: hipLaunchKernelGGL(mb_memeff_write, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, nq); break;
+        case 9: hipLaunchKernelGGL(mb_memeff_both, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq); break;
+        case 10: hipLaunchKernelGGL(mb_write1, dim3((uint32_t)grid64), dim3(64), lds, stream, P, nq); break;
+        case 11: hipLaunchKernelGGL(mb_write3_temporal, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq); break;
+        case 12: hipLaunchKernelGGL(mb_write3_bursts, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, nq); break;
+        case 13: hipLaunchKernelGGL(mb_oneshot_x4, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq); break;
+        default: return -1;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+}  // extern "C"

@@ -209,7 +209,7 @@ class TensorListPlan:
                 self._handle = ctypes.c_void_p()
 
     def __del__(self):  # pragma: no cover - interpreter shutdown order is not ours to test
-        if sys.is_finalizing():
+        if sys is None or sys.is_finalizing():
             return  # the process is ending: nothing to give back, and the runtime underneath may be half gone
         try:
             self.close()

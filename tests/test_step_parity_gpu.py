@@ -865,3 +865,72 @@ def test_c5_llama7b_pure_fp16_with_overflow_injection(oracle, cuda_device):
             nonfinite = sum(int((~torch.isfinite(v)).sum().item()) for v in V)
             assert nonfinite > 0
         del before
+
+
+def test_c5_llama7b_dynamic_scaling_through_the_optimizer(oracle, cuda_device):
+    """The Llama-7B configuration at its real size through ``Adam(precision=PURE_FP16)``: a clean step, a step in which
+    one gradient element in 10^6 is 6e4 (the stored second moment overflows: flag read back, optimizer-state scale halved,
+    m and v of ALL 291 tensors zeroed, adam.py:278-288), then a clean step at the halved scale.  Windows of several
+    tensors are re-computed by the oracle with the scale and the step count the optimizer used; the scale trajectory
+    is exact; after the backoff there is no non-zero m or v anywhere."""
+    from fairscale_amd.optim import Adam, Precision
+
+    dev = cuda_device
+    free, _total = torch.cuda.mem_get_info(dev)
+    need = 6_738_415_616 * 8 + (8 << 30)
+    if free < need:
+        pytest.skip(f"needs {need >> 30} GiB of device memory, {free >> 30} GiB free")
+    shapes = C.llama7b_shapes()
+    sizes = [C.numel(s) for s in shapes]
+    gen = torch.Generator(device=dev).manual_seed(5050)
+    params = [torch.empty(sh, device=dev, dtype=torch.float16).normal_(0, 0.02, generator=gen).requires_grad_() for sh in shapes]
+    clean = [torch.empty(sh, device=dev, dtype=torch.float16).normal_(0, 1e-3, generator=gen) for sh in shapes]
+    opt = Adam(params, lr=1e-3, precision=Precision.PURE_FP16)
+    assert opt._optim_scale == 65536.0
+    probe = [0, 1, 5, 8, 9, 145, 289, 290]  # embedding, attention, ffn, norm vectors, head
+    rng = np.random.default_rng(5052)
+    want_scale = {1: 65536.0, 2: 65536.0, 3: 32768.0}  # the scale each step runs with
+    for step in (1, 2, 3):
+        for t, p in enumerate(params):
+            p.grad = clean[t].clone() if step == 2 else clean[t]
+            if step == 2 and sizes[t] >= 1_000_000:  # 1 element in 10^6, seeded
+                idx = torch.from_numpy(rng.integers(0, sizes[t], size=sizes[t] // 1_000_000)).to(dev)
+                p.grad.view(-1)[idx] = 6e4
+        zero = torch.zeros(1, device=dev, dtype=torch.float16)
+        before = {}
+        for t in probe:
+            st = opt.state[params[t]] if step > 1 else {}
+            flat = params[t].detach().view(-1)
+            before[t] = {"p": flat.clone(), "m": st["exp_avg"].view(-1).clone() if st else zero.expand(sizes[t]).clone(),
+                         "v": st["exp_avg_sq"].view(-1).clone() if st else zero.expand(sizes[t]).clone()}
+        scale = opt._optim_scale
+        assert scale == want_scale[step]
+        print(f"[c5 optimizer] step {step} at scale {scale}", flush=True)
+        opt.step()
+        torch.cuda.synchronize()
+        kw = dict(DEFAULT, step=step, optim_scale=scale)
+        for t in probe:
+            n = sizes[t]
+            wins = [(0, n)] if n <= 65536 else _windows(n, 3, 65536, 5200 + t)
+            st = opt.state[params[t]]
+            if step == 2:
+                # m and v were zeroed after the kernel had stored them: only the parameters can be compared, and they
+                # come from the unrounded fp32 moments, overflow or not (fused_adam_cuda_kernel.cu:106-112)
+                flag = np.zeros(1, np.float32)
+                for lo, hi in wins:
+                    p, m, v = (before[t][k][lo:hi].cpu().numpy().copy() for k in ("p", "m", "v"))
+                    oracle.step_c(PURE16, p, m, v, params[t].grad.view(-1)[lo:hi].cpu().numpy(), None, found_inf=flag, **kw)
+                    assert C.assert_close(params[t].detach().view(-1)[lo:hi].cpu().numpy(), p, f"C5 optimizer step 2 tensor {t} p[{lo}:{hi}]") == 0
+            else:
+                after = {"p": params[t].detach().view(-1), "m": st["exp_avg"].view(-1), "v": st["exp_avg_sq"].view(-1)}
+                f = _window_check(oracle, PURE16, before[t], after, params[t].grad.view(-1), wins, kw, f"C5 optimizer step {step} tensor {t}")
+                assert f == 0.0
+        if step == 2:
+            assert opt._optim_scale == 32768.0 and opt._steps_since_optim_scale_change == 0
+            for p in params:
+                st = opt.state[p]
+                assert not bool(st["exp_avg"].any()) and not bool(st["exp_avg_sq"].any()), "state not zeroed after the overflow"
+                assert st["step"] == 2
+        del before
+    assert opt._optim_scale == 32768.0 and opt._steps_since_optim_scale_change == 1
+    assert all(opt.state[p]["step"] == 3 for p in params)
