@@ -19,7 +19,8 @@ FULL_PRECISION_FP16_COPY = 4
 
 ABI_VERSION = 3
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
+# $FSADAM_LIBRARY names another build of the same ABI (the measurement variants of csrc/build.py); normally unset
+_LIB_PATH = os.environ.get("FSADAM_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
 
 
 class FsAdamTensor(ctypes.Structure):

@@ -33,18 +33,25 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
-def build_library(verbose: bool = False) -> str:
-    """Always recompiles; returns the path of the shared library."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", INCLUDE, "-I", HERE, "-o", LIBRARY + ".tmp", SOURCE]
+APPROX_LIBRARY = os.path.join(HERE, "libfsadam_approx.so")
+
+
+def build_library(verbose: bool = False, experiment_approx: bool = False) -> str:
+    """Always recompiles; returns the path of the shared library.  ``experiment_approx``: build the measurement
+    variant with approximate division and square root into ``libfsadam_approx.so`` instead (never loaded by the
+    package unless ``FSADAM_LIBRARY`` names it; its results are NOT bit-identical to the oracle)."""
+    target = APPROX_LIBRARY if experiment_approx else LIBRARY
+    extra = ["-DFSADAM_EXPERIMENT_APPROX_DIV_SQRT"] if experiment_approx else []
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra, "-I", INCLUDE, "-I", HERE, "-o", target + ".tmp", SOURCE]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"  # the host pass does not know the device feature
     log = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
-    os.replace(LIBRARY + ".tmp", LIBRARY)
+    os.replace(target + ".tmp", target)
     if verbose and log.strip():
         print(log, file=sys.stderr)
-    return LIBRARY
+    return target
 
 
 MEMBENCH_SOURCE = os.path.join(HERE, "membench.hip")
@@ -103,6 +110,9 @@ def build_rows_module(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
+    if "--experiment-approx" in sys.argv[1:]:
+        print(build_library(verbose=True, experiment_approx=True))
+        sys.exit(0)
     print(build_library(verbose=True))
     print(build_membench(verbose=True))
     print(build_rows_module(verbose=True))

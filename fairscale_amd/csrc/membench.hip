@@ -217,6 +217,50 @@ __global__ __launch_bounds__(64) void mb_oneshot_x4(f4* p_, f4* m_, f4* v_, cons
     for (int k = 0; k < 4; ++k) st<true>(p + k * 64, a[k]);
 }
 
+// ---- variants 14/15: one-shot tiles in an XCD-aware order.  Workgroup b runs on XCD b % 8 (hardware dispatch is
+// round-robin over the eight XCDs); within every group of 8 * R workgroups, workgroup b takes tile
+// (b % 8) * R + (b / 8) % R, so that each XCD (each L2) works through runs of R consecutive tiles.
+__device__ __forceinline__ int64_t xcd_tile(int64_t b, int log2_run) {
+    const int64_t span = (int64_t)8 << log2_run, group = b / span, in = b % span;
+    return group * span + ((in & 7) << log2_run) + (in >> 3);
+}
+__global__ __launch_bounds__(64) void mb_oneshot_xcd(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq, int log2_run) {
+    const int64_t i = xcd_tile(blockIdx.x, log2_run) * 64 + threadIdx.x;
+    if (i >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + i;
+    f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+       d = ld<true>((FS_GLOBAL const f4*)g_ + i);
+    fake_update(a, b, c, d);
+    st<true>(m, b);
+    st<true>(v, c);
+    st<true>(p, a);
+}
+__global__ __launch_bounds__(64) void mb_memeff_both_xcd(f2* p_, f4* m_, f4* v_, const f2* g_, int64_t n4, int log2_run) {
+    const int64_t i = xcd_tile(blockIdx.x, log2_run) * 64 + threadIdx.x;
+    if (i >= n4) return;
+    f2 a = ld<true>((FS_GLOBAL const f2*)p_ + i);
+    const f2 d = ld<true>((FS_GLOBAL const f2*)g_ + i);
+    f4 b = ld<true>((FS_GLOBAL const f4*)m_ + i), c = ld<true>((FS_GLOBAL const f4*)v_ + i);
+    const f4 g = {d[0], d[1], d[0], d[1]};
+    b = b * 0.9f + g * 0.1f;
+    c = c * 0.999f + g * g * 0.001f;
+    a[0] -= b[0] * 0.001f;
+    a[1] -= b[1] * 0.001f;
+    st<true>((FS_GLOBAL f4*)m_ + i, b);
+    st<true>((FS_GLOBAL f4*)v_ + i, c);
+    st<true>((FS_GLOBAL f2*)p_ + i, a);
+}
+__global__ __launch_bounds__(64) void mb_write3_xcd(f4* p_, f4* m_, f4* v_, int64_t nq, int log2_run) {
+    const int64_t i = xcd_tile(blockIdx.x, log2_run) * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    st<true>((FS_GLOBAL f4*)m_ + i, val);
+    st<true>((FS_GLOBAL f4*)v_ + i, val);
+    st<true>((FS_GLOBAL f4*)p_ + i, val);
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
 __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -240,7 +284,7 @@ int64_t fsadam_membench_table_bytes(int64_t numel) {
 
 // Launches variant `kind` once over `numel` elements (a multiple of 4) on `stream`.  p, m, v, g: device buffers of
 // numel floats (the MEMORY_EFFICIENT variants use the first half of p and g as fp16).  lds_bytes: untouched LDS given to
-// every workgroup (caps residency).  param: variant 1: workgroups per compute unit.  table: device memory of
+// every workgroup (caps residency).  param: variant 1: workgroups per compute unit; variants 14-16: log2 of the run length in tiles.  table: device memory of
 // fsadam_membench_table_bytes(numel) bytes for variants 3, 4 and -1 (-1 fills it; do that once before them).
 // Returns 0, or -1 for an unknown kind / bad argument, -2 for a launch error.
 int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t numel, int lds_bytes, int param, void* table, void* sink,
@@ -286,6 +330,18 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
         case 11: hipLaunchKernelGGL(mb_write3_temporal, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq); break;
         case 12: hipLaunchKernelGGL(mb_write3_bursts, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, nq); break;
         case 13: hipLaunchKernelGGL(mb_oneshot_x4, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq); break;
+        case 14:
+        case 15:
+        case 16: {
+            if (param < 0 || param > 24) return -1;
+            const int64_t span = (int64_t)8 << param;
+            const int64_t grid = (grid64 + span - 1) / span * span;  // whole groups: the surplus workgroups find no tile
+            if (grid > 0x7ffffff0) return -1;
+            if (kind == 14) hipLaunchKernelGGL(mb_oneshot_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, G, nq, param);
+            else if (kind == 15) hipLaunchKernelGGL(mb_memeff_both_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq, param);
+            else hipLaunchKernelGGL(mb_write3_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, nq, param);
+            break;
+        }
         default: return -1;
     }
     return hipGetLastError() == hipSuccess ? 0 : -2;

@@ -36,3 +36,23 @@ def test_bytes_per_parameter_follow_from_the_streams():
             "MEMORY_EFFICIENT_MIXED_PRECISION": (2 + 4 + 4 + 2) + (2 + 4 + 4), "PURE_FP16": 4 * 2 + 3 * 2}
     assert bench.BYTES_PER_PARAM == want
     assert bench.HBM_PEAK_GBS == 8000.0
+
+
+def test_spread_is_min_median_max():
+    import bench
+
+    assert bench.spread([3.0, 1.0, 2.0]) == {"min": 1.0, "median": 2.0, "max": 3.0}
+    assert bench.spread([4.0, 1.0, 2.0, 3.0]) == {"min": 1.0, "median": 2.5, "max": 4.0}
+
+
+def test_benchmark_configurations_have_the_sizes_the_baseline_names():
+    """The lists bench.py builds for configurations 2 and 5 are the ones the parity tests use."""
+    import inspect
+
+    import bench
+    import _cases as C
+
+    src = inspect.getsource(bench.measure_c2) + inspect.getsource(bench.measure_c5)
+    assert "124_439_808" in src and "6_738_415_616" in src and "== 148" in src and "== 291" in src
+    assert sum(C.numel(s) for s in C.gpt2_small_shapes()) == 124_439_808 and len(C.gpt2_small_shapes()) == 148
+    assert sum(C.numel(s) for s in C.llama7b_shapes()) == 6_738_415_616 and len(C.llama7b_shapes()) == 291
