@@ -81,6 +81,7 @@ SIGNATURES = {
     "fsadam_plan_step_dev_scale": (_i32, [_vp, _f32, _f32, _f32, _f32, _vp, _f32, _f32, _i32, _i32, _i32, _vp, _vp]),
     "fsadam_plan_info": (_i32, [_vp, ctypes.POINTER(FsAdamPlanInfo)]),
     "fsadam_plan_lazy_events": (_i32, [_vp, _i32]),
+    "fsadam_plan_zero_state": (_i32, [_vp, _vp]),
     "fsadam_plan_destroy": (_i32, [_vp]),
     "fsadam_head_elems": (_i32, [ctypes.POINTER(FsAdamTensor), _i32, ctypes.POINTER(_i64)]),
     "fsadam_layout": (_i32, [ctypes.POINTER(FsAdamTensor), _i64, _i32, ctypes.POINTER(FsAdamLayout), ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_uint8)]),

@@ -219,4 +219,33 @@ __global__ __launch_bounds__(BLOCK) void fsadam_tiles(const ChunkDesc* __restric
     if (ModeTraits<MODE>::kScaled && bad != 0) *(gptr<float>)found_inf = 1.0f;
 }
 
+// m = v = 0 over every tile of a step's table (same layout, same tile size): what follows an overflow of the fp16
+// state (fairscale/optim/adam.py:285-288) in one launch, instead of a foreach over hundreds of tensors.
+template <int MODE, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void fsadam_zero_state(const ChunkDesc* __restrict__ table, TileMap map) {
+    using S = typename ModeTraits<MODE>::S;
+    constexpr int E = ModeTraits<MODE>::kElems;
+    constexpr uint32_t kTile = BLOCK * E;
+    uint32_t chunk, off;
+    locate_tile(map, blockIdx.x, kTile, chunk, off);
+    typedef uint32_t desc_words_t __attribute__((ext_vector_type(16)));
+    const desc_words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) desc_words_t*>(
+        (const __attribute__((address_space(4))) ChunkDesc*)table + chunk);
+    const ChunkDesc d = __builtin_bit_cast(ChunkDesc, raw);
+    if (off >= d.n) return;
+    const uint32_t left = d.n - off;
+    gptr<S> m = (gptr<S>)d.m + off;
+    gptr<S> v = (gptr<S>)d.v + off;
+    if (left >= kTile) {
+        typename VecOf<S, E>::type zero = {};
+        store_vec<S, E>(m + threadIdx.x * E, zero);
+        store_vec<S, E>(v + threadIdx.x * E, zero);
+    } else {
+        for (uint32_t e = threadIdx.x; e < left; e += BLOCK) {
+            m[e] = (S)0;
+            v[e] = (S)0;
+        }
+    }
+}
+
 }  // namespace

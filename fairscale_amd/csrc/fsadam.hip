@@ -620,6 +620,29 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     return mark_use(slot.mark, stream, plan->lazy_events);
 }
 
+// m = v = 0 for every tensor of the plan's current table: one launch over the step's own layout.
+int plan_zero_state(FsAdamPlan* plan, hipStream_t stream) {
+    if (plan->rows.empty() || plan->current < 0) return fail(FSADAM_EINVAL, "plan has no tensors; call fsadam_plan_set_tensors first");
+    if (int refused = refuse_capture(stream)) return refused;
+    int dev = -1;
+    FS_HIP(hipGetDevice(&dev));
+    if (dev != plan->device)
+        return fail(FSADAM_EINVAL, "plan belongs to device " + std::to_string(plan->device) + ", current device is " + std::to_string(dev));
+    const Layout& L = plan->layout;
+    const int64_t n_blocks = L.blocks();
+    if (n_blocks == 0) return FSADAM_OK;
+    TableSlot& slot = plan->slots[plan->current];
+    int rc = mark_order_after(slot.mark, stream);
+    if (rc) return rc;
+    const size_t lds = 32768;  // a pass that only writes runs best with few waves per compute unit
+    if (plan->mode == FSADAM_PURE_FP16)
+        hipLaunchKernelGGL((fsadam_zero_state<FSADAM_PURE_FP16, kBlock>), dim3((uint32_t)n_blocks), dim3(kBlock), lds, stream, slot.d_table, tile_map(L));
+    else
+        hipLaunchKernelGGL((fsadam_zero_state<FSADAM_FULL_PRECISION, kBlock>), dim3((uint32_t)n_blocks), dim3(kBlock), lds, stream, slot.d_table, tile_map(L));
+    FS_HIP(hipGetLastError());
+    return mark_use(slot.mark, stream, plan->lazy_events);
+}
+
 
 // ---- gradient pass, host side -----------------------------------------------------------------
 
@@ -1073,6 +1096,11 @@ int fsadam_plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float
     if (!plan) return fail(FSADAM_EINVAL, "plan is NULL");
     return plan_step(plan, lr, beta1, beta2, eps, grad_scale, nullptr, optim_scale, decay, step, eps_mode, bias_correction,
                      found_inf_dev, static_cast<hipStream_t>(hip_stream));
+}
+
+int fsadam_plan_zero_state(FsAdamPlan* plan, void* hip_stream) {
+    if (!plan) return fail(FSADAM_EINVAL, "plan is NULL");
+    return plan_zero_state(plan, static_cast<hipStream_t>(hip_stream));
 }
 
 int fsadam_plan_step_dev_scale(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, const float* grad_scale_dev,

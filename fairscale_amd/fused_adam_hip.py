@@ -262,6 +262,21 @@ class TensorListPlan:
                 _cabi.check(L.fsadam_plan_step(self._handle, lr, beta1, beta2, eps, float(grad_scale), optim_scale, decay,
                                                int(step), int(eps_mode), int(bias_correction), flag, stream))
 
+    def current(self) -> bool:
+        """The device table holds the rows of the last step (nothing failed or was left half-written since)."""
+        return self._rows is not None and not self._dirty
+
+    def holds_state(self, exp_avg_ptrs: List[int], exp_avg_sq_ptrs: List[int]) -> bool:
+        """Does the device table point at exactly these m and v tensors, in this order?"""
+        rows = self._rows
+        return (self.current() and rows.shape[0] == len(exp_avg_ptrs) == len(exp_avg_sq_ptrs)
+                and rows[:, 1].tolist() == exp_avg_ptrs and rows[:, 2].tolist() == exp_avg_sq_ptrs)
+
+    def zero_state(self) -> None:
+        """m = v = 0 for every tensor of the last step's list, in one launch (fsadam_plan_zero_state)."""
+        with _on_device(self.device):
+            _cabi.check(_cabi.lib().fsadam_plan_zero_state(self._handle, _stream_handle(self.device)))
+
     def step(self, tensor_lists: Sequence[Sequence[torch.Tensor]], lr: float, beta1: float, beta2: float, eps: float,
              grad_scale: float, optim_scale: float, found_inf: Optional[torch.Tensor], step: int, eps_mode: int,
              bias_correction: int, decay: float) -> None:

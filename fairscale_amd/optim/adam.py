@@ -607,9 +607,33 @@ class Adam(torch.optim.Optimizer):
         gradient yet, which the reference gives state here as well."""
         stale: List[torch.Tensor] = []
         created = False
+        # The parameters of the step that has just run are zeroed through its own table, one launch per group and
+        # device: the state tensors the table points at are the ones the step checked and used.
+        done = set()
+        for gi, group in enumerate(self.param_groups):
+            cache = self._steady_group(gi, group)  # None when the list, the state map or the master copies changed since
+            if cache is None:
+                continue
+            states, device = cache[2], cache[5]
+            plan = self._plans.get((gi, device))
+            active = [st for st in states if st is not None]
+            if plan is None or not plan.current() or len(states) != len(group["params"]):
+                continue
+            # the table must still point at these very tensors (a group that has not stepped yet in this call was
+            # gathered a step ago): compare the pointers it was built from with the state tensors of now
+            try:
+                now = [[st["exp_avg"].data_ptr() for st in active], [st["exp_avg_sq"].data_ptr() for st in active]]
+            except KeyError:
+                continue
+            if not plan.holds_state(now[0], now[1]):
+                continue
+            plan.zero_state()
+            done.update(id(st) for st in active)
         for group in self.param_groups:
             for p in group["params"]:
                 state = self.state[p]
+                if id(state) in done:
+                    continue
                 for key in ("exp_avg", "exp_avg_sq"):
                     t = state.get(key)
                     if t is not None and t.dtype == self.optim_type and t.shape == p.shape and t.device == p.device:

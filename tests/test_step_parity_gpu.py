@@ -934,3 +934,47 @@ def test_c5_llama7b_dynamic_scaling_through_the_optimizer(oracle, cuda_device):
         del before
     assert opt._optim_scale == 32768.0 and opt._steps_since_optim_scale_change == 1
     assert all(opt.state[p]["step"] == 3 for p in params)
+
+
+@pytest.mark.parametrize("mode", [FULL, MIXED, MEMEFF, PURE16])
+def test_zero_state_clears_m_and_v_and_nothing_else(cuda_device, mode):
+    """``fsadam_plan_zero_state``: m = v = 0 for every tensor of the plan (sizes around every boundary, views that start
+    between cache lines), the bytes around each state tensor, the parameters and the gradients untouched."""
+    from fairscale_amd import fused_adam_hip
+
+    sizes = [1, 7, 255, 256, 257, 4095, 4096, 4097, 8191, 16385, 70001, 131072, 131073, 300001, 0, 5]
+    host = C.Tensors(mode, sizes, 5400 + mode)
+    for arrs in (host.m, host.v):
+        for a in arrs:
+            a[...] = 3.0
+    dev = GpuList(host, cuda_device, misalign={"m": 3, "v": 1, "p": 1})
+    # sentinels around the state views: _place puts a view `k` elements into an allocation 8 elements longer than needed
+    guards = []
+    for lst, k in ((dev.m, 3), (dev.v, 1)):
+        for t in lst:
+            base = t._base if t._base is not None else t
+            base[:k] = 7.0
+            base[k + t.numel():] = 7.0
+            guards.append((base, k, t.numel()))
+    grads = to_gpu(host.grads(1), cuda_device)
+    lists = [dev.p, dev.m, dev.v, grads] + ([dev.p16] if mode == MIXED else [])
+    before_p = [t.clone() for t in dev.p]
+    before_g = [t.clone() for t in grads]
+    plan = fused_adam_hip.TensorListPlan(mode, cuda_device)
+    with pytest.raises(Exception, match="no tensors"):
+        plan.zero_state()
+    plan.step(lists, 1e-3, 0.9, 0.999, 1e-8, 1.0, 65536.0 if mode == PURE16 else 1.0, dev.found_inf, 1, 1, 1, 0.0)
+    after_p = [t.clone() for t in dev.p]
+    assert any(bool(t.any()) for t in dev.m)
+    plan.zero_state()
+    torch.cuda.synchronize(cuda_device)
+    for t in dev.m + dev.v:
+        assert not bool(t.any())
+    for base, k, n in guards:
+        assert bool((base[:k] == 7.0).all()) and bool((base[k + n:] == 7.0).all()), "zero_state wrote outside a state tensor"
+    for a, b in zip(after_p, dev.p):
+        assert torch.equal(a, b)
+    for a, b in zip(before_g, grads):
+        assert torch.equal(a, b)
+    assert not all(torch.equal(a, b) for a, b in zip(before_p, dev.p))  # the step itself had run
+    plan.close()
