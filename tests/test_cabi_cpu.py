@@ -285,6 +285,37 @@ def test_rows_that_continue_each_other_are_laid_out_as_one_run():
     assert layout(rows4, _cabi.FULL_PRECISION)[0]["n_runs"] == 1
 
 
+def test_shared_chunks_shrink_until_they_divide_the_tensors_well():
+    """The chunk a shared descriptor covers starts at half the smallest large tensor and is halved while the tiles behind
+    the tensors' ends (workgroups that are launched and find nothing to do) exceed 1 % of the elements."""
+    import _cases as C
+
+    A = 0x7000_0000_0000
+    row = lambda n: (A, A + (1 << 40), A + (2 << 40), A + (3 << 40), A + (4 << 40), n)  # noqa: E731
+    old = _cabi.get_option("merge_runs")
+    _cabi.set_option("merge_runs", 0)  # every row has the same fake address: keep them apart
+    try:
+        # Llama-7B: 2^23 would leave the last chunk of every 4096 x 11008 matrix 5/8 empty; 2^20 divides every matrix
+        sizes = [C.numel(sh) for sh in C.llama7b_shapes()]
+        lay, _, _ = layout([row(n) for n in sizes], _cabi.PURE_FP16)
+        assert lay["large_chunk_elems"] == 1 << 20
+        large = [n for n in sizes if n >= 131072]
+        assert lay["grid_large"] * lay["tile_elems"] == sum(large)  # not one tile behind an end
+        # GPT-2 small: every matrix is a multiple of 65536 elements except the embedding
+        sizes = [C.numel(sh) for sh in C.gpt2_small_shapes()]
+        lay, _, _ = layout([row(n) for n in sizes], _cabi.MIXED_PRECISION)
+        large = [n for n in sizes if n >= 131072]
+        assert lay["large_chunk_elems"] == 65536 and lay["grid_large"] * lay["tile_elems"] - sum(large) < 0.01 * sum(large)
+        # the flat shard keeps the largest chunk: 98 x 2^24 is 0.87 % more than 1.63e9
+        lay, _, _ = layout([row(1_630_000_000)], _cabi.MEMORY_EFFICIENT_MIXED_PRECISION)
+        assert lay["large_chunk_elems"] == 1 << 24 and lay["n_large_descriptors"] == 98
+        # one tensor just over a power of two: 2^24 + 2^20 elements would need two chunks of 2^23... halved down to 2^20
+        lay, _, _ = layout([row((1 << 24) + (1 << 20))], _cabi.FULL_PRECISION)
+        assert lay["large_chunk_elems"] == 1 << 20 and lay["n_large_descriptors"] == 17
+    finally:
+        _cabi.set_option("merge_runs", old)
+
+
 def test_layout_counts_heads_among_the_small_descriptors(two_classes):
     A = 0x7000_0000_0000
     t = lambda n, off: (A + off, A + (1 << 34) + off, A + (2 << 34) + off, A + (3 << 34) + off, 0, n)  # noqa: E731
@@ -333,6 +364,9 @@ def test_layout_matches_a_python_model_on_drawn_lists():
             if large:
                 chunk = 1 << ((min(large) // 2).bit_length() - 1)
             chunk = min(cap, max(65536, min(1 << 24, chunk)))
+            # halved until the tiles behind the tensors' ends are at most 1 % of the large tensors' elements
+            while chunk > 65536 and (sum(-(-n // chunk) * chunk for n in large) - sum(large)) * 100 > sum(large):
+                chunk //= 2
             want_large = sum(-(-n // chunk) for n in large)
             # a middle class only for 2..64 tiles per descriptor and chunks of at most half the large threshold
             mid_chunk = tile * mid_tiles if mid_tiles > 1 and 2 * tile * mid_tiles <= 131072 else 0
