@@ -190,11 +190,18 @@ int64_t head_elems(const FsAdamTensor& r, int mode, const Options& opt) {
         return c;
     };
     int64_t best = 0, best_cost = cost(0);
+    if (best_cost == 0) return 0;  // every stream on a 1 KiB boundary already
+    int64_t tried[10];
+    int n_tried = 0;
     for (const Stream& st : streams) {
         if (!st.ptr) continue;
         for (uintptr_t boundary : {uintptr_t(128), uintptr_t(1024)}) {
             const uintptr_t a = reinterpret_cast<uintptr_t>(st.ptr);
             const int64_t head = (int64_t)(((boundary - (a & (boundary - 1))) & (boundary - 1)) / st.size);
+            bool seen = head == 0;  // streams that are off by the same amount propose the same heads
+            for (int k = 0; k < n_tried && !seen; ++k) seen = tried[k] == head;
+            if (seen) continue;
+            tried[n_tried++] = head;
             const int64_t c = cost(head);
             if (c < best_cost || (c == best_cost && head < best)) { best = head; best_cost = c; }
         }
@@ -284,16 +291,23 @@ void build_runs(const FsAdamTensor* tensors, int64_t n, int mode, bool merge, st
     }
 }
 
-// `runs`: the rows build_runs made (none empty).
-Layout compute_layout(const std::vector<FsAdamTensor>& runs, int mode, const Options& opt) {
+// The head of every run, computed once per table (it is asked for three times on the way to one).
+void compute_heads(const std::vector<FsAdamTensor>& runs, int mode, const Options& opt, std::vector<int64_t>& heads) {
+    heads.resize(runs.size());
+    for (size_t k = 0; k < runs.size(); ++k) heads[k] = head_elems(runs[k], mode, opt);
+}
+
+// `runs`: the rows build_runs made (none empty); `heads`: compute_heads of them.
+Layout compute_layout(const std::vector<FsAdamTensor>& runs, const std::vector<int64_t>& heads, int mode, const Options& opt) {
     Layout L;
     L.tile_elems = kBlock * mode_elems(mode);
     L.mid_chunk_elems = mid_chunk_for(L.tile_elems, opt.mid_tiles);
     L.n_runs = (int64_t)runs.size();
     int64_t min_large = 0;
-    for (const FsAdamTensor& r : runs) {
+    for (size_t k = 0; k < runs.size(); ++k) {
+        const FsAdamTensor& r = runs[k];
         L.total_elems += r.numel;
-        const int64_t head = head_elems(r, mode, opt), body = r.numel - head;
+        const int64_t head = heads[k], body = r.numel - head;
         (row_vector_ok(r, mode, head) ? L.n_vector : L.n_scalar) += 1;
         const int cls = class_of(body, L);
         if (cls == kClassLarge) {
@@ -310,16 +324,16 @@ Layout compute_layout(const std::vector<FsAdamTensor>& runs, int mode, const Opt
     // chunk of every 4096 x 11008 matrix 5/8 empty, 7 % of all workgroups; 2^20 divides every matrix of the list)
     for (; L.large_chunk_elems > kMinLargeChunk; L.large_chunk_elems /= 2) {
         int64_t body_total = 0, padded_total = 0;
-        for (const FsAdamTensor& r : runs) {
-            const int64_t body = r.numel - head_elems(r, mode, opt);
+        for (size_t k = 0; k < runs.size(); ++k) {
+            const int64_t body = runs[k].numel - heads[k];
             if (class_of(body, L) != kClassLarge) continue;
             body_total += body;
             padded_total += ceil_div(body, L.large_chunk_elems) * L.large_chunk_elems;
         }
         if ((padded_total - body_total) * 100 <= body_total) break;
     }
-    for (const FsAdamTensor& r : runs) {
-        const int64_t head = head_elems(r, mode, opt), body = r.numel - head;
+    for (size_t k = 0; k < runs.size(); ++k) {
+        const int64_t head = heads[k], body = runs[k].numel - head;
         L.n_small_descs += ceil_div(head, L.tile_elems);
         const int cls = class_of(body, L);
         if (cls == kClassLarge) L.n_large_descs += ceil_div(body, L.large_chunk_elems);
@@ -365,6 +379,7 @@ struct FsAdamPlan {
     Layout layout;
     std::vector<FsAdamTensor> rows;  // what the current table was built from
     std::vector<FsAdamTensor> runs;  // scratch of plan_set_tensors: the rows after merging
+    std::vector<int64_t> heads;      // ... and the head of each
     bool lazy_events = false;        // see UseMark; fsadam_plan_lazy_events
     int64_t uploads = 0;
     TableSlot slots[kTableSlots];
@@ -542,7 +557,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     }
     if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
     build_runs(tensors, n, plan->mode, plan->opt.merge_runs != 0, plan->runs, nullptr);
-    Layout L = compute_layout(plan->runs, plan->mode, plan->opt);
+    compute_heads(plan->runs, plan->mode, plan->opt, plan->heads);
+    Layout L = compute_layout(plan->runs, plan->heads, plan->mode, plan->opt);
     for (int64_t t = 0; t < n; ++t) L.n_empty += tensors[t].numel == 0 ? 1 : 0;
     const int64_t n_descs = L.descs();
     if (L.blocks() > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
@@ -571,8 +587,9 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     ChunkDesc* large = slot.h_table;
     ChunkDesc* mid = large + L.n_large_descs;
     ChunkDesc* small = mid + L.n_mid_descs;
-    for (const FsAdamTensor& r : plan->runs) {
-        const int64_t head = head_elems(r, plan->mode, plan->opt), body = r.numel - head;
+    for (size_t k = 0; k < plan->runs.size(); ++k) {
+        const FsAdamTensor& r = plan->runs[k];
+        const int64_t head = plan->heads[k], body = r.numel - head;
         small += fill_descs(small, r, plan->mode, 0, head, L.tile_elems);
         const int cls = class_of(body, L);
         if (cls == kClassLarge) large += fill_descs(large, r, plan->mode, head, body, L.large_chunk_elems);
@@ -1049,7 +1066,9 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
     std::vector<FsAdamTensor> runs;
     std::vector<int64_t> run_of;
     build_runs(tensors, n_tensors, precision_mode, opt.merge_runs != 0, runs, &run_of);
-    const Layout L = compute_layout(runs, precision_mode, opt);
+    std::vector<int64_t> heads;
+    compute_heads(runs, precision_mode, opt, heads);
+    const Layout L = compute_layout(runs, heads, precision_mode, opt);
     out->tile_elems = L.tile_elems;
     out->large_chunk_elems = L.large_chunk_elems;
     out->n_large_tensors = L.n_large;
@@ -1068,7 +1087,7 @@ int fsadam_layout(const FsAdamTensor* tensors, int64_t n_tensors, int precision_
         if (tensors[t].numel == 0) out->n_empty_tensors += 1;
         // a tensor is laid out with the run it belongs to
         const FsAdamTensor* run = run_of[(size_t)t] >= 0 ? &runs[(size_t)run_of[(size_t)t]] : nullptr;
-        const int64_t head = run ? head_elems(*run, precision_mode, opt) : 0;
+        const int64_t head = run ? heads[(size_t)run_of[(size_t)t]] : 0;
         if (tensor_class) tensor_class[t] = run ? (uint8_t)class_of(run->numel - head, L) : 0;
         if (vector_ok) vector_ok[t] = (run && row_vector_ok(*run, precision_mode, head)) ? 1 : 0;
     }

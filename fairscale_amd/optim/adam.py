@@ -73,13 +73,18 @@ def _adjacent_runs(tensors: List[torch.Tensor]) -> List[List[int]]:
     memory (entry k+1 starts at the byte behind entry k's last element)."""
     runs: List[List[int]] = []
     end = None
+    last = None  # the last non-empty tensor of the current run
     for k, t in enumerate(tensors):
+        if t.numel() == 0 and runs:
+            runs[-1].append(k)  # nothing to place: it rides along (the native layout skips empty rows as well)
+            continue
         ptr = t.data_ptr()
-        if end is not None and ptr == end and t.is_contiguous() and t.dtype == tensors[k - 1].dtype and t.device == tensors[k - 1].device:
+        if end is not None and ptr == end and t.is_contiguous() and t.dtype == last.dtype and t.device == last.device:
             runs[-1].append(k)
         else:
             runs.append([k])
         end = ptr + t.numel() * t.element_size() if t.is_contiguous() else None
+        last = t
     return runs
 
 

@@ -1,0 +1,74 @@
+"""Host logic that lays optimizer state out like the parameters (``fairscale_amd/optim/adam.py``), on CPU tensors: which
+parameters form a run, where a stream that accompanies a run has to start, and when existing state counts as in place.
+The reference allocates ``zeros_like`` per parameter (``fairscale/optim/adam.py:226-228``); parameters that are
+back-to-back views of one buffer are what OSS makes of a rank's shard (``fairscale/optim/oss.py:630-659``)."""
+from __future__ import annotations
+
+import torch
+
+from fairscale_amd.optim import adam as A
+
+
+def _views(flat, sizes, lead=0):
+    out, at = [], lead
+    for n in sizes:
+        out.append(flat[at:at + n])
+        at += n
+    return out
+
+
+def test_adjacent_runs_follow_the_memory_not_the_list():
+    flat = torch.zeros(100_000)
+    a, b, c, d = _views(flat, [10, 7, 5000, 3], lead=1)
+    other = torch.zeros(7)
+    assert A._adjacent_runs([a, b, c, d]) == [[0, 1, 2, 3]]
+    assert A._adjacent_runs([a, other, c, d]) == [[0], [1], [2, 3]]            # a stranger in the middle
+    assert A._adjacent_runs([a, c, d]) == [[0], [1, 2]]                         # b left out (a frozen parameter): a gap
+    assert A._adjacent_runs([b, a]) == [[0], [1]]                               # the wrong way round
+    assert A._adjacent_runs([a, b.double(), c]) == [[0], [1], [2]]              # another dtype in between breaks the run
+    two_d = flat[6000:6000 + 12].view(3, 4)
+    tail = flat[6012:6020]
+    assert A._adjacent_runs([two_d, tail]) == [[0, 1]]                          # shapes do not matter, bytes do
+    assert A._adjacent_runs([two_d.t(), tail]) == [[0], [1]]                    # a non-contiguous tensor is a run of its own
+    assert A._adjacent_runs([]) == []
+    empty = flat[10:10]
+    assert A._adjacent_runs([flat[1:10], empty, flat[10:20]]) == [[0, 1, 2]]    # an empty view continues the run
+
+
+def test_a_stream_for_a_run_starts_where_the_run_leaves_its_cache_line():
+    flat = torch.zeros(200_000)  # float32: 512 elements = 2 KiB
+    base = flat.data_ptr() // 4
+    for lead in (1, 3, 31, 100, 511, 513):
+        first = flat[lead:lead + 50_000]
+        if first.data_ptr() % 128 == 0:
+            continue
+        for dtype in (torch.float32, torch.float16):
+            buf = A._buffer_placed_like(first, 50_000, dtype, zero=True)
+            assert buf.numel() == 50_000 and buf.dtype == dtype and buf.is_contiguous() and not bool(buf.any())
+            # same element offset modulo 512: one head length aligns both
+            assert (buf.data_ptr() // buf.element_size()) % 512 == (base + lead) % 512
+    # short runs and runs that start on a line get a plain allocation
+    short = flat[1:1 + 100]
+    assert A._buffer_placed_like(short, 100, torch.float32, zero=True).numel() == 100
+    on_line = (-(flat.data_ptr() // 4)) % 32  # host allocations are only 64-byte aligned: find a 128-byte boundary
+    assert not A._needs_offset(short, 100) and not A._needs_offset(flat[on_line:on_line + 50_000], 50_000)
+    assert A._needs_offset(flat[on_line + 1:on_line + 50_001], 50_000)
+
+
+def test_state_counts_as_placed_only_when_it_follows_the_parameters():
+    params = torch.zeros(60_000)
+    state = torch.zeros(60_000 + 512)
+    sizes = [9000, 20, 30_000]
+    lead = 3
+    likes = _views(params, sizes, lead=lead)
+    want = (likes[0].data_ptr() // 4) % 512
+    start = (want - (state.data_ptr() // 4) % 512) % 512
+    good = _views(state, sizes, lead=start)
+    assert A._placed(good, likes)
+    assert not A._placed(_views(state, sizes, lead=(start + 1) % 512), likes)            # packed, at another offset
+    assert not A._placed([torch.zeros(n) for n in sizes], likes)                          # one allocation each
+    assert not A._placed([good[0], good[1], torch.zeros(sizes[2])], likes)               # the last one elsewhere
+    assert not A._placed([good[0], good[1], good[2][:-1]], likes)                         # a size that does not fit
+    # a short run, or one that starts on a line: packed is enough
+    small_likes = _views(params, [10, 20], lead=1)
+    assert A._placed(_views(state, [10, 20], lead=7), small_likes)
