@@ -256,6 +256,110 @@ def test_random_lists_match_the_oracle(oracle, cuda_device, seed):
              optim_scale=optim_scale, mutate=plant)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_packed_lists_match_the_oracle(oracle, cuda_device, seed):
+    """Drawn lists whose streams are packed into flat buffers: every stream starts a drawn number of elements into its
+    buffer (the same for all streams or one per stream, so that heads differ), and at drawn places a stream skips a few
+    elements or a tensor of one stream lives in an allocation of its own, which cuts the list into runs of drawn lengths
+    (single tensors, short runs, runs that are large only together).  Sizes around the tile, the shared-descriptor and
+    the large-tensor boundaries, empty tensors inside runs.  Two steps against the oracle, and the run count against a
+    count made here."""
+    import random
+
+    from fairscale_amd import fused_adam_hip
+
+    rng = random.Random(12000 + seed)
+    mode = rng.choice([FULL, MIXED, MEMEFF, PURE16])
+    tile = 512 if mode == PURE16 else 256
+    pd, gd, sd = C.MODE_DTYPES[mode]
+
+    def draw_size():
+        kind = rng.randrange(7)
+        if kind == 0:
+            return rng.choice([0, 1, 2, 3])
+        if kind == 1:
+            return rng.randrange(4, tile)
+        if kind == 2:
+            return tile * rng.randrange(1, 40) + rng.choice([-1, 0, 1])
+        if kind == 3:
+            return rng.randrange(tile, 9000)
+        if kind == 4:
+            return rng.randrange(9000, 70000)
+        if kind == 5:
+            return 131072 + rng.choice([-1, 0, 1, 255])
+        return rng.randrange(131072, 400000)
+
+    sizes = [draw_size() for _ in range(rng.randrange(2, 40))]
+    if sum(sizes) == 0:
+        sizes.append(300)
+    names = ["p", "m", "v", "g"] + (["p16"] if mode == MIXED else [])
+    same_lead = rng.randrange(2) == 0
+    lead0 = rng.choice([0, 1, 3, 64, 130, 511])
+    lead = {name: (lead0 if same_lead else rng.choice([0, 1, 3, 64, 130, 511])) for name in names}
+    # where a stream breaks: ("gap", name, tensor) skips 1-70 elements in front of the tensor; ("own", name, tensor) puts it elsewhere
+    breaks = {}
+    for t in range(1, len(sizes)):
+        if rng.random() < 0.25:
+            breaks[(rng.choice(names), t)] = rng.choice(["gap", "own"])
+    host = C.Tensors(mode, sizes, 12100 + seed)
+    dtype_of = {"p": host.p[0].dtype if sizes else pd, "m": sd, "v": sd, "g": gd, "p16": np.float16}
+
+    def pack(arrs, name):
+        dt = TORCH_DTYPE[np.dtype(dtype_of[name])]
+        flat = torch.full((sum(sizes) + lead[name] + 80 * len(sizes) + 8,), 7.0, dtype=dt, device=cuda_device)
+        out, at = [], lead[name]
+        for t, a in enumerate(arrs):
+            how = breaks.get((name, t))
+            if how == "gap":
+                at += 1 + (t * 13 + seed) % 70
+            view = torch.empty(a.size, dtype=dt, device=cuda_device) if how == "own" else flat[at:at + a.size]
+            view.copy_(torch.from_numpy(a))
+            out.append(view)
+            if how != "own":
+                at += a.size
+        return out
+
+    dev = GpuList.__new__(GpuList)
+    dev.mode, dev.device, dev.misalign = mode, cuda_device, {}
+    dev.p, dev.m, dev.v = pack(host.p, "p"), pack(host.m, "m"), pack(host.v, "v")
+    dev.p16 = pack(host.p16, "p16") if host.p16 is not None else None
+    dev.found_inf = torch.zeros(1, dtype=torch.float32, device=cuda_device)
+    hyper = dict(lr=rng.choice([1e-3, 3e-2]), beta1=rng.choice([0.9, 0.5]), beta2=rng.choice([0.999, 0.95]), eps=rng.choice([1e-8, 1e-3]),
+                 eps_mode=rng.randrange(2), bias_correction=rng.randrange(2), decay=rng.choice([0.0, 0.01]))
+    grad_scale = rng.choice([1.0, 128.0, 3.0]) if mode != FULL else rng.choice([1.0, 3.0])
+    optim_scale = rng.choice([65536.0, 1000.0]) if mode == PURE16 else 1.0
+    # runs as the library must see them: a new one wherever any stream breaks in front of a non-empty tensor
+    want_runs, open_run, broken = 0, False, False
+    for t, n in enumerate(sizes):
+        # a gap in front of a tensor stays in the stream whatever the tensor's size; an allocation of its own breaks the
+        # sequence in front of and behind that tensor, unless the tensor is empty (an empty row is skipped)
+        broken = (broken or any(breaks.get((name, t)) == "gap" for name in names)
+                  or (n > 0 and any(breaks.get((name, t)) == "own" for name in names))
+                  or (t > 0 and sizes[t - 1] > 0 and any(breaks.get((name, t - 1)) == "own" for name in names)))
+        if n == 0:
+            continue
+        if not open_run or broken:
+            want_runs += 1
+        open_run, broken = True, False
+    print(f"seed {seed}: mode {mode}, {len(sizes)} tensors, {sum(sizes)} elements, leads {lead}, {len(breaks)} breaks, {want_runs} runs", flush=True)
+    plan = fused_adam_hip.TensorListPlan(mode, cuda_device)
+    flag = np.zeros(1, np.float32)
+    for step in (1, 2):
+        grads = host.grads(step, scale=grad_scale)
+        g = pack(grads, "g")
+        lists = [dev.p, dev.m, dev.v, g] + ([dev.p16] if mode == MIXED else [])
+        kw = dict(hyper, step=step, grad_scale=grad_scale, optim_scale=optim_scale)
+        plan.step(lists, kw["lr"], kw["beta1"], kw["beta2"], kw["eps"], grad_scale, optim_scale, dev.found_inf, step, kw["eps_mode"],
+                  kw["bias_correction"], kw["decay"])
+        torch.cuda.synchronize(cuda_device)
+        oracle_step(oracle, host, grads, flag, **kw)
+        compare(host, dev, f"packed draw {seed} mode={mode} step={step}")
+        # (fewer when the allocator happens to put two of the separately allocated tensors back to back)
+        assert 1 <= plan.info()["n_runs"] <= want_runs
+    assert float(dev.found_inf.item()) == float(flag[0])
+    plan.close()
+
+
 def test_pure_fp16_odd_optim_scale_rounds_twice_on_every_path(oracle, cuda_device):
     """m and v are stored as half(float32(m' * S)): two roundings (kernel.cu:100-101).  With a scale that is
     not a power of two the float32 product is inexact, and about one element in 10^4 lands exactly between
