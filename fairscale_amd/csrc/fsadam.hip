@@ -20,13 +20,13 @@
 //     128 bits per lane for fp32 streams and 64 or 128 bits per lane for fp16 streams, all with
 //     the non-temporal hint (nothing is re-read).
 // The tensor list becomes a device-resident table of 64-byte chunk descriptors (five pointers
-// already advanced to the chunk, element count, alignment flag), uploaded once and reused every
-// step.  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
+// already advanced to the chunk, element count), uploaded once and reused every step.  Consecutive
+// tensors that continue each other in every stream are laid out as one (build_runs).  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
 // tile = block & (2^k - 1).  Large tensors share one descriptor among 2^k tiles, middle-sized ones
 // among 16, small ones get one descriptor per tile, each class placed after the one before, so ONE
 // launch covers any number of tensors (the reference needs a launch per 36 tensors / 320 chunks
-// because its table travels by value in the kernel arguments).  Ragged tiles (the end of a tensor) take an element-wise path with the same
-// arithmetic; full tiles of a tensor whose streams are only element-aligned use the same vector
+// because its table travels by value in the kernel arguments).  Ragged tiles (the end of a tensor)
+// take an element-wise path with the same arithmetic; full tiles of a tensor whose streams are only element-aligned use the same vector
 // instructions at odd addresses.
 //
 // Arithmetic is IEEE float32 exactly as written in the reference source: separate multiplies and
@@ -346,12 +346,12 @@ Layout compute_layout(const std::vector<FsAdamTensor>& runs, const std::vector<i
 }  // namespace
 
 // "Everything enqueued so far that uses X" as something a stream or the host can wait for.  By default
-// the event is recorded right behind every use.  With option "lazy_events" it is only recorded when
+// the event is recorded right behind every use.  A plan that was told so (fsadam_plan_lazy_events) records it only when
 // somebody needs it (another stream takes over, the table slot is about to be overwritten, the plan
 // goes away), so that a step on the stream of the step before enqueues its kernel and nothing else
 // (3 us less per step); recording late marks a later point of the same stream, which covers the uses
 // as well, but it touches the stream after the call that used it has returned: the caller must then
-// keep every stream it has passed alive for as long as the plan (or the cache) lives.
+// keep every stream it has passed to that plan alive for as long as the plan lives.
 struct UseMark {
     hipEvent_t event = nullptr;
     hipStream_t stream = nullptr;  // where the uses were enqueued
