@@ -59,6 +59,8 @@ def parse_args():
                          "traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--micro", action="store_true", help="run the structure microbenchmarks instead (needs libfsadam_membench.so) and print a table")
     ap.add_argument("--micro-numel", type=int, default=SHARD_NUMEL)
+    ap.add_argument("--micro-data", default="random", choices=["random", "zeros"],
+                    help="what the microbenchmark's buffers hold and its write-only kernels store (the bandwidth of this part depends on it)")
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (lds_throttle, merge_runs, align_heads, mid_tiles, ...)")
     return ap.parse_args()
 
@@ -446,8 +448,14 @@ def run_micro(torch, args, device):
     L.fsadam_membench_launch.argtypes = [i32, vp, vp, vp, vp, i64, i32, i32, vp, vp, vp]
     L.fsadam_membench_table_bytes.restype = i64
     L.fsadam_membench_table_bytes.argtypes = [i64]
+    L.fsadam_membench_set_pattern.restype = None
+    L.fsadam_membench_set_pattern.argtypes = [i32]
+    L.fsadam_membench_set_pattern(1 if args.micro_data == "random" else 0)
     n = args.micro_numel // 4 * 4
     bufs = [torch.zeros(n, device=device, dtype=torch.float32) for _ in range(4)]
+    if args.micro_data == "random":  # values like a step's: every mantissa bit in use (the update keeps them bounded)
+        for b in bufs:
+            b.normal_(0, 1.0)
     table = torch.zeros(L.fsadam_membench_table_bytes(n), device=device, dtype=torch.uint8)
     sink = torch.zeros(1, device=device)
     stream = torch.cuda.current_stream().cuda_stream
@@ -476,7 +484,7 @@ def run_micro(torch, args, device):
                         "ms_median": sp["median"], "ms_min": sp["min"], "gbs_at_median": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
         print(f"{name:<78s} {sp['median']:8.3f} ms  {gbs:7.0f} GB/s  {gbs / HBM_PEAK_GBS * 100:5.1f} %", flush=True)
 
-    print(f"# {n} elements per stream; GB/s of algorithmic bytes at the median of 10 launches; peak {HBM_PEAK_GBS:.0f} GB/s")
+    print(f"# {n} elements per stream; GB/s of algorithmic bytes at the median of 10 launches; peak {HBM_PEAK_GBS:.0f} GB/s; data: {args.micro_data}")
     print("# fp32 shape: p, m, v, g read, p, m, v written (28 B/element)")
     for wg in (4, 8, 16):
         measure(f"grid-stride loop, 256 threads, {wg} workgroups per CU, non-temporal", 1, 28, param=wg)
@@ -515,7 +523,7 @@ def run_micro(torch, args, device):
     w_gbs = by["writes only (10 B/element), ballast 12288 B"]["gbs_at_median"]
     serial = 22.0 / (12.0 / r_gbs + 10.0 / w_gbs)
     print(f"# 12 B read at {r_gbs:.0f} GB/s + 10 B written at {w_gbs:.0f} GB/s, one after the other: {serial:.0f} GB/s = {serial / HBM_PEAK_GBS * 100:.1f} % of peak")
-    print(json.dumps({"micro": results, "numel": n, "memeff_mix_ceiling_gbs": serial}))
+    print(json.dumps({"micro": results, "numel": n, "data": args.micro_data, "memeff_mix_ceiling_gbs": serial}))
 
 
 def main():

@@ -26,6 +26,20 @@ __device__ __forceinline__ void st(FS_GLOBAL T* p, T v) {
     else *p = v;
 }
 
+// What the write-only kernels store: zeros, or (pattern != 0) floats in [1, 2) whose mantissa bits are a hash of the
+// position -- the bandwidth of this part depends on the data (see run_micro in bench.py), and optimizer state is not zeros.
+__device__ __forceinline__ f4 fill_value(int64_t i, int pattern) {
+    if (!pattern) return f4{0.f, 0.f, 0.f, 0.f};
+    uint32_t h = (uint32_t)i * 2654435761u + 0x9e3779b9u;
+    f4 out;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        out[k] = __builtin_bit_cast(float, (h & 0x007fffffu) | 0x3f800000u);
+    }
+    return out;
+}
+
 // the stand-in for the update: enough arithmetic to keep every loaded value alive, nothing more
 __device__ __forceinline__ void fake_update(f4& p, f4& m, f4& v, f4 g) {
     m = m * 0.9f + g * 0.1f;
@@ -123,10 +137,10 @@ __global__ __launch_bounds__(64) void mb_read4(const f4* p_, const f4* m_, const
                  ld<true>((FS_GLOBAL const f4*)g_ + i);
     if (s[0] + s[1] + s[2] + s[3] == 12345.678f) *sink = 1.0f;  // never true for the zero-filled buffers: keeps the loads
 }
-__global__ __launch_bounds__(64) void mb_write3(f4* p_, f4* m_, f4* v_, int64_t nq) {
+__global__ __launch_bounds__(64) void mb_write3(f4* p_, f4* m_, f4* v_, int64_t nq, int pattern) {
     const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
     if (i >= nq) return;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f4 val = fill_value(i, pattern);
     st<true>((FS_GLOBAL f4*)m_ + i, val);
     st<true>((FS_GLOBAL f4*)v_ + i, val);
     st<true>((FS_GLOBAL f4*)p_ + i, val);
@@ -141,11 +155,11 @@ __global__ __launch_bounds__(64) void mb_memeff_read(const f2* p_, const f4* m_,
     const f4 s = ld<true>((FS_GLOBAL const f4*)m_ + i) + ld<true>((FS_GLOBAL const f4*)v_ + i);
     if (s[0] + s[1] + s[2] + s[3] + a[0] + a[1] + d[0] + d[1] == 12345.678f) *sink = 1.0f;
 }
-__global__ __launch_bounds__(64) void mb_memeff_write(f2* p_, f4* m_, f4* v_, int64_t n4) {
+__global__ __launch_bounds__(64) void mb_memeff_write(f2* p_, f4* m_, f4* v_, int64_t n4, int pattern) {
     const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
     if (i >= n4) return;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
-    const f2 half = {0.f, 0.f};
+    const f4 val = fill_value(i, pattern);
+    const f2 half = {val[0], val[1]};
     st<true>((FS_GLOBAL f4*)m_ + i, val);
     st<true>((FS_GLOBAL f4*)v_ + i, val);
     st<true>((FS_GLOBAL f2*)p_ + i, half);
@@ -170,23 +184,23 @@ __global__ __launch_bounds__(64) void mb_memeff_both(f2* p_, f4* m_, f4* v_, con
 // 10: ONE stream written (a fill); 11: three streams with plain (temporal) stores; 12: three streams, every wave
 // writes four consecutive vectors per stream (4 KiB bursts); 13: the 28-byte shape with four vectors per lane and
 // stream: all sixteen loads first, then all twelve stores (longer same-direction bursts per wave).
-__global__ __launch_bounds__(64) void mb_write1(f4* p_, int64_t nq) {
+__global__ __launch_bounds__(64) void mb_write1(f4* p_, int64_t nq, int pattern) {
     const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
     if (i >= nq) return;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f4 val = fill_value(i, pattern);
     st<true>((FS_GLOBAL f4*)p_ + i, val);
 }
-__global__ __launch_bounds__(64) void mb_write3_temporal(f4* p_, f4* m_, f4* v_, int64_t nq) {
+__global__ __launch_bounds__(64) void mb_write3_temporal(f4* p_, f4* m_, f4* v_, int64_t nq, int pattern) {
     const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
     if (i >= nq) return;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f4 val = fill_value(i, pattern);
     st<false>((FS_GLOBAL f4*)m_ + i, val);
     st<false>((FS_GLOBAL f4*)v_ + i, val);
     st<false>((FS_GLOBAL f4*)p_ + i, val);
 }
-__global__ __launch_bounds__(64) void mb_write3_bursts(f4* p_, f4* m_, f4* v_, int64_t nq) {
+__global__ __launch_bounds__(64) void mb_write3_bursts(f4* p_, f4* m_, f4* v_, int64_t nq, int pattern) {
     const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f4 val = fill_value(base, pattern);
 #pragma unroll
     for (int k = 0; k < 4; ++k) if (base + k * 64 < nq) st<true>((FS_GLOBAL f4*)m_ + base + k * 64, val);
 #pragma unroll
@@ -252,10 +266,10 @@ __global__ __launch_bounds__(64) void mb_memeff_both_xcd(f2* p_, f4* m_, f4* v_,
     st<true>((FS_GLOBAL f4*)v_ + i, c);
     st<true>((FS_GLOBAL f2*)p_ + i, a);
 }
-__global__ __launch_bounds__(64) void mb_write3_xcd(f4* p_, f4* m_, f4* v_, int64_t nq, int log2_run) {
+__global__ __launch_bounds__(64) void mb_write3_xcd(f4* p_, f4* m_, f4* v_, int64_t nq, int log2_run, int pattern) {
     const int64_t i = xcd_tile(blockIdx.x, log2_run) * 64 + threadIdx.x;
     if (i >= nq) return;
-    const f4 val = {0.f, 0.f, 0.f, 0.f};
+    const f4 val = fill_value(i, pattern);
     st<true>((FS_GLOBAL f4*)m_ + i, val);
     st<true>((FS_GLOBAL f4*)v_ + i, val);
     st<true>((FS_GLOBAL f4*)p_ + i, val);
@@ -274,7 +288,14 @@ __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, u
 
 }  // namespace
 
+namespace {
+int g_pattern = 0;
+}
+
 extern "C" {
+
+// What the write-only variants store from now on: 0 zeros (default), 1 floats with hashed mantissas.
+void fsadam_membench_set_pattern(int pattern) { g_pattern = pattern != 0; }
 
 // Bytes the caller must provide for the descriptor table of variants 3 and 4 (chunks of 2^16 quads).
 int64_t fsadam_membench_table_bytes(int64_t numel) {
@@ -322,13 +343,13 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
             break;
         }
         case 5: hipLaunchKernelGGL(mb_read4, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq, (float*)sink); break;
-        case 6: hipLaunchKernelGGL(mb_write3, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq); break;
+        case 6: hipLaunchKernelGGL(mb_write3, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq, g_pattern); break;
         case 7: hipLaunchKernelGGL(mb_memeff_read, dim3((uint32_t)grid64), dim3(64), lds, stream, (const f2*)p, M, V, (const f2*)g, nq, (float*)sink); break;
-        case 8: hipLaunchKernelGGL(mb_memeff_write, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, nq); break;
+        case 8: hipLaunchKernelGGL(mb_memeff_write, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, nq, g_pattern); break;
         case 9: hipLaunchKernelGGL(mb_memeff_both, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq); break;
-        case 10: hipLaunchKernelGGL(mb_write1, dim3((uint32_t)grid64), dim3(64), lds, stream, P, nq); break;
-        case 11: hipLaunchKernelGGL(mb_write3_temporal, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq); break;
-        case 12: hipLaunchKernelGGL(mb_write3_bursts, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, nq); break;
+        case 10: hipLaunchKernelGGL(mb_write1, dim3((uint32_t)grid64), dim3(64), lds, stream, P, nq, g_pattern); break;
+        case 11: hipLaunchKernelGGL(mb_write3_temporal, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, nq, g_pattern); break;
+        case 12: hipLaunchKernelGGL(mb_write3_bursts, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, nq, g_pattern); break;
         case 13: hipLaunchKernelGGL(mb_oneshot_x4, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq); break;
         case 14:
         case 15:
@@ -339,7 +360,7 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
             if (grid > 0x7ffffff0) return -1;
             if (kind == 14) hipLaunchKernelGGL(mb_oneshot_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, G, nq, param);
             else if (kind == 15) hipLaunchKernelGGL(mb_memeff_both_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq, param);
-            else hipLaunchKernelGGL(mb_write3_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, nq, param);
+            else hipLaunchKernelGGL(mb_write3_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, nq, param, g_pattern);
             break;
         }
         default: return -1;
