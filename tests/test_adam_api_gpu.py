@@ -487,7 +487,7 @@ def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_
     head aligns every stream; the values must be those of the same parameters allocated one by one, and
     saving and loading the state must keep them."""
     Adam, _, Precision = api
-    sizes = (9001, 33, 8192, 140003, 20000)
+    sizes = (9001, 33, 0, 8192, 140003, 20000)  # an empty parameter rides along in the run
     separate = _random_problem(precision_name, cuda_device, sizes)
     dtype = separate[0].dtype
     flat = torch.empty(sum(sizes) + 3, device=cuda_device, dtype=dtype)

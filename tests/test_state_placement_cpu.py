@@ -72,3 +72,14 @@ def test_state_counts_as_placed_only_when_it_follows_the_parameters():
     # a short run, or one that starts on a line: packed is enough
     small_likes = _views(params, [10, 20], lead=1)
     assert A._placed(_views(state, [10, 20], lead=7), small_likes)
+
+
+def test_empty_parameters_inside_a_run_do_not_unsettle_it():
+    params = torch.zeros(1000)
+    state = torch.zeros(1000)
+    likes = [params[0:100], params[100:100], params[100:300]]
+    assert A._adjacent_runs(likes) == [[0, 1, 2]]
+    placed = [state[0:100], state[100:100], state[100:300]]
+    assert A._placed(placed, likes)
+    assert A._placed([state[0:100], torch.zeros(0), state[100:300]], likes)     # wherever the empty one "lies"
+    assert not A._placed([state[0:100], state[100:100], state[101:301]], likes)
