@@ -264,7 +264,9 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
  * when it writes back: at least 1.07e9 elements in every case; a tensor of 131072 elements or more takes one
  * descriptor per 2^16..2^24 elements, smaller ones up to 16, plus one for a misaligned start).  Tuning options
  * are not consulted.  All calls on one GPU share that GPU's array: calls whose kernels may overlap (different
- * streams without an order between them, or two threads) race; calls on one stream are ordered by it. */
+ * streams without an order between them, or two threads) race; calls on one stream are ordered by it.  The call may
+ * be recorded into a HIP graph (its scalars do not depend on a step count); make the first call on a device outside
+ * any capture, since that call looks up the array's address. */
 #define FSADAM_NOALLOC_MAX_DESCRIPTORS 4096
 #define FSADAM_NOALLOC_MAX_WORKGROUPS 65536
 int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int grad_dtype, float inv_scale, const float* inv_scale_dev,

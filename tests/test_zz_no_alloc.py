@@ -124,3 +124,50 @@ def test_lists_beyond_the_scratch_are_refused(cuda_device):
     rc = L.fsadam_grad_pass_noalloc(rows, 1, _cabi.GRAD_F32, 0.5, None, 1, None, None, None, None)
     assert rc == -1 and b"workgroups" in L.fsadam_last_error()
     torch.cuda.synchronize()
+
+
+def test_recorded_into_a_graph_and_replayed(cuda_device):
+    """What the entry point is for: between the begin and the end of a capture nothing may allocate.  One call outside
+    any capture first (it looks the array's address up), then the call is recorded and replayed four times on fresh
+    gradients, with eager work and synchronisations in between; every replay against ``fsadam_grad_pass`` run eagerly
+    on copies."""
+    from fairscale_amd import _cabi
+
+    L = _cabi.lib()
+    sizes = [300_001, 70_000, 5, 4096]
+    gen = torch.Generator(device="cpu").manual_seed(9)
+    grads = [torch.randn(n, generator=gen).half().to(cuda_device) for n in sizes]
+    rows = _rows(grads)
+    flag = torch.zeros(1, device=cuda_device)
+    ssq = torch.zeros(1, device=cuda_device, dtype=torch.float64)
+    amax = torch.zeros(1, device=cuda_device)
+
+    def call(stream):
+        _cabi.check(L.fsadam_grad_pass_noalloc(rows, len(grads), _cabi.GRAD_F16, 0.5, None, 1, flag.data_ptr(), ssq.data_ptr(), amax.data_ptr(), stream))
+
+    side = torch.cuda.Stream(cuda_device)
+    with torch.cuda.stream(side):
+        call(side.cuda_stream)
+    torch.cuda.synchronize(cuda_device)
+    graph = torch.cuda.CUDAGraph()
+    print("[noalloc] capture", flush=True)
+    with torch.cuda.graph(graph, stream=side):
+        call(torch.cuda.current_stream(cuda_device).cuda_stream)
+    torch.cuda.synchronize(cuda_device)
+    for rep in range(4):
+        fresh = [torch.randn(n, generator=gen).half().to(cuda_device) for n in sizes]
+        if rep == 2:
+            fresh[1][123] = float("inf")
+        for t, f in zip(grads, fresh):
+            t.copy_(f)
+        flag.zero_()
+        torch.cuda.synchronize(cuda_device)
+        print(f"[noalloc] replay {rep}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize(cuda_device)
+        want = _call("fsadam_grad_pass", fresh, 0.5, True)
+        assert flag.item() == want[0] == (1.0 if rep == 2 else 0.0)
+        assert amax.item() == want[2]
+        assert abs(ssq.item() - want[1]) <= 1e-6 * abs(want[1]) or ssq.item() == want[1]
+        for t, f in zip(grads, fresh):
+            assert np.array_equal(_bits(t), _bits(f)), f"replay {rep}"
