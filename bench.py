@@ -434,8 +434,8 @@ def load_traffic(workload_key):
 def run_micro(torch, args, device):
     """The measurements the kernel's shape rests on, from kernels the tree builds (fairscale_amd/csrc/membench.hip):
     one-shot tiles against a grid-stride loop, residency (LDS ballast) sweep, temporal against non-temporal accesses,
-    the descriptor read with one scalar load against a descriptor staged in LDS, and the ceilings of this part for reads
-    only, writes only and the step's mix.  Prints one line per variant and one JSON line at the end."""
+    the descriptor read with one scalar load against a descriptor staged in LDS, tiles in an XCD-aware order, reads and
+    writes in device-wide phases, and the ceilings of this part for reads only, writes only and the step's mix.  Prints one line per variant and one JSON line at the end."""
     import ctypes
 
     path = os.path.join(REPO, "fairscale_amd", "csrc", "libfsadam_membench.so")
@@ -518,6 +518,9 @@ def run_micro(torch, args, device):
     measure("reads and writes (22 B/element), ballast 12288 B", 9, 22, lds=12288)
     for lg in (2, 10):
         measure(f"reads and writes (22 B/element), runs of {1 << lg:5d} tiles per XCD, ballast 12288 B", 15, 22, lds=12288, param=lg)
+    print("# reads and writes in device-wide phases set by the real-time counter: every wave loads only in the first 12/22 of a period, stores only in the rest")
+    for lds, period in ((0, 50), (0, 200), (8192, 50), (8192, 200), (12288, 50), (12288, 200)):
+        measure(f"reads and writes (22 B/element), phases of {period / 100:.1f} us, ballast {lds:5d} B", 19, 22, lds=lds, param=period)
     by = {r["variant"]: r for r in results}
     r_gbs = by["reads only (12 B/element), ballast 12288 B"]["gbs_at_median"]
     w_gbs = by["writes only (10 B/element), ballast 12288 B"]["gbs_at_median"]

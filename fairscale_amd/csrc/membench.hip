@@ -275,6 +275,77 @@ __global__ __launch_bounds__(64) void mb_write3_xcd(f4* p_, f4* m_, f4* v_, int6
     st<true>((FS_GLOBAL f4*)p_ + i, val);
 }
 
+// ---- variants 17/18/19: device-wide read and write phases set by the clock.  Every wave reads the constant-rate real-time
+// counter (the same for all waves of the device), issues its loads only in the first `split` ticks of every `period` ticks and
+// its stores only in the rest, so that at any instant the whole device moves data in one direction.  Waits are bounded.
+__device__ __forceinline__ void wait_phase(uint32_t period, uint32_t split, bool writing) {
+    for (int spin = 0; spin < 100000; ++spin) {
+        const uint32_t t = (uint32_t)(wall_clock64() % period);
+        if ((t >= split) == writing) return;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+__global__ __launch_bounds__(64) void mb_oneshot_phased(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq, uint32_t period, uint32_t split) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + i;
+    wait_phase(period, split, false);
+    f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+       d = ld<true>((FS_GLOBAL const f4*)g_ + i);
+    fake_update(a, b, c, d);
+    // the wait must not be hoisted above the loads' return: it depends on a loaded value
+    if (a[0] == 12345.678f) return;
+    wait_phase(period, split, true);
+    st<true>(m, b);
+    st<true>(v, c);
+    st<true>(p, a);
+}
+__global__ __launch_bounds__(64) void mb_oneshot_x4_phased(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq, uint32_t period, uint32_t split) {
+    const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (base + 192 >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + base;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + base;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + base;
+    FS_GLOBAL const f4* g = (FS_GLOBAL const f4*)g_ + base;
+    f4 a[4], b[4], c[4], d[4];
+    wait_phase(period, split, false);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        a[k] = ld<true>((FS_GLOBAL const f4*)p + k * 64); b[k] = ld<true>((FS_GLOBAL const f4*)m + k * 64);
+        c[k] = ld<true>((FS_GLOBAL const f4*)v + k * 64); d[k] = ld<true>(g + k * 64);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fake_update(a[k], b[k], c[k], d[k]);
+    if (a[0][0] + a[1][0] + a[2][0] + a[3][0] == 12345.678f) return;
+    wait_phase(period, split, true);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(m + k * 64, b[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(v + k * 64, c[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st<true>(p + k * 64, a[k]);
+}
+__global__ __launch_bounds__(64) void mb_memeff_both_phased(f2* p_, f4* m_, f4* v_, const f2* g_, int64_t n4, uint32_t period, uint32_t split) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    wait_phase(period, split, false);
+    f2 a = ld<true>((FS_GLOBAL const f2*)p_ + i);
+    const f2 d = ld<true>((FS_GLOBAL const f2*)g_ + i);
+    f4 b = ld<true>((FS_GLOBAL const f4*)m_ + i), c = ld<true>((FS_GLOBAL const f4*)v_ + i);
+    const f4 g = {d[0], d[1], d[0], d[1]};
+    b = b * 0.9f + g * 0.1f;
+    c = c * 0.999f + g * g * 0.001f;
+    a[0] -= b[0] * 0.001f;
+    a[1] -= b[1] * 0.001f;
+    if (a[0] == 12345.678f) return;
+    wait_phase(period, split, true);
+    st<true>((FS_GLOBAL f4*)m_ + i, b);
+    st<true>((FS_GLOBAL f4*)v_ + i, c);
+    st<true>((FS_GLOBAL f2*)p_ + i, a);
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
 __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -305,7 +376,7 @@ int64_t fsadam_membench_table_bytes(int64_t numel) {
 
 // Launches variant `kind` once over `numel` elements (a multiple of 4) on `stream`.  p, m, v, g: device buffers of
 // numel floats (the MEMORY_EFFICIENT variants use the first half of p and g as fp16).  lds_bytes: untouched LDS given to
-// every workgroup (caps residency).  param: variant 1: workgroups per compute unit; variants 14-16: log2 of the run length in tiles.  table: device memory of
+// every workgroup (caps residency).  param: variant 1: workgroups per compute unit; variants 14-16: log2 of the run length in tiles; variants 17-19: the period in 10 ns ticks.  table: device memory of
 // fsadam_membench_table_bytes(numel) bytes for variants 3, 4 and -1 (-1 fills it; do that once before them).
 // Returns 0, or -1 for an unknown kind / bad argument, -2 for a launch error.
 int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t numel, int lds_bytes, int param, void* table, void* sink,
@@ -361,6 +432,17 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
             if (kind == 14) hipLaunchKernelGGL(mb_oneshot_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, G, nq, param);
             else if (kind == 15) hipLaunchKernelGGL(mb_memeff_both_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq, param);
             else hipLaunchKernelGGL(mb_write3_xcd, dim3((uint32_t)grid), dim3(64), lds, stream, P, M, V, nq, param, g_pattern);
+            break;
+        }
+        case 17:
+        case 18:
+        case 19: {
+            // param: the period in 10 ns ticks of the real-time counter; loads get the share of it that they have of the bytes
+            if (param < 2 || param > 100000) return -1;
+            const uint32_t period = (uint32_t)param, split = kind == 19 ? period * 12 / 22 : period * 16 / 28;
+            if (kind == 17) hipLaunchKernelGGL(mb_oneshot_phased, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq, period, split);
+            else if (kind == 18) hipLaunchKernelGGL(mb_oneshot_x4_phased, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq, period, split);
+            else hipLaunchKernelGGL(mb_memeff_both_phased, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq, period, split);
             break;
         }
         default: return -1;
