@@ -33,8 +33,7 @@ __device__ __forceinline__ typename VecOf<T, E>::type load_vec(gptr<const T> ptr
 }
 template <typename T, int E>
 __device__ __forceinline__ void store_vec(gptr<T> ptr, typename VecOf<T, E>::type value) {
-    using V = typename VecOf<T, E>::in_memory;
-    __builtin_nontemporal_store(value, reinterpret_cast<gptr<V>>(ptr));
+    store_through((gptr<void>)ptr, value);
 }
 
 // Two packed halves in one 32-bit word: non-zero when either is +-inf or NaN (exponent field all

@@ -97,13 +97,14 @@ struct Options {
     int64_t merge_runs = 1;         // 1: consecutive tensors that continue each other in every stream are laid out as one
 };
 
-// Residency that measured fastest with one wave64 per workgroup and one vector per lane per stream:
-// about 40-48 KiB of loads in flight per compute unit, i.e. 10 waves of the 4 KiB-per-wave modes and
-// 12-13 of the 3-4 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
+// Residency that measured fastest with one wave64 per workgroup, one vector per lane per stream and stores that
+// are written through (store_through): about 40 KiB of loads in flight per compute unit, i.e. 10 waves of the
+// 4 KiB-per-wave modes and 13 of the 2-3 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
+// Each value is the middle of a plateau about 1 KiB wide either way; 2 KiB off costs 2-8 points.
 int64_t default_lds_throttle(int mode) {
     switch (mode) {
-        case FSADAM_FULL_PRECISION: return 16384;
-        case FSADAM_FULL_PRECISION_FP16_COPY: return 16384;
+        case FSADAM_FULL_PRECISION: return 15360;
+        case FSADAM_FULL_PRECISION_FP16_COPY: return 15360;
         case FSADAM_MIXED_PRECISION: return 15360;
         case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
         default: return 12288;

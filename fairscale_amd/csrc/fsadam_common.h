@@ -72,6 +72,30 @@ struct StepScalars {
 template <typename T>
 using gptr = FS_GLOBAL T*;
 
+#ifdef __HIPCC__
+// One 8- or 16-byte store that leaves for memory as it is issued: device scope (sc1: the L2 writes it through
+// instead of keeping a dirty line to evict later) and non-temporal.  The compiler's non-temporal store sets nt
+// alone; with sc1 as well a kernel that reads and writes streams moves 2 points more of the HBM rate (measured
+// on this part with every combination of the three policy bits, on the loads and on the stores).  Nothing reads
+// these bytes again before the kernel ends, so the scope costs nothing.  The address may be any (unaligned-access
+// mode), the value any type of 8 or 16 bytes.
+// The instruction comes from inline assembly (no builtin sets this combination of bits), so the compiler does not
+// see a store: it neither counts it (harmless: waiting for a count that leaves the older loads out still waits for
+// them) nor keeps its hands off the data registers for the two wait states this target needs between a store of
+// more than 64 bits and a vector instruction that overwrites its data -- the s_nop does.
+template <typename V>
+__device__ __forceinline__ void store_through(gptr<void> ptr, V value) {
+    static_assert(sizeof(V) == 8 || sizeof(V) == 16, "one dwordx2 or dwordx4");
+    if constexpr (sizeof(V) == 16) {
+        typedef uint32_t words_t __attribute__((ext_vector_type(4)));
+        asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(ptr), "v"(__builtin_bit_cast(words_t, value)) : "memory");
+    } else {
+        typedef uint32_t words_t __attribute__((ext_vector_type(2)));
+        asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(ptr), "v"(__builtin_bit_cast(words_t, value)) : "memory");
+    }
+}
+#endif
+
 template <int MODE>
 struct ModeTraits;
 template <>

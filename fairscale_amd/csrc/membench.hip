@@ -346,6 +346,71 @@ __global__ __launch_bounds__(64) void mb_memeff_both_phased(f2* p_, f4* m_, f4* 
     st<true>((FS_GLOBAL f2*)p_ + i, a);
 }
 
+// ---- variants 20/21: the cache-policy bits of the memory instructions.  gfx950 loads and stores carry three bits: sc0 and
+// sc1 (the scope the access must be coherent at: wave, workgroup, device, system) and nt (non-temporal); the compiler's
+// non-temporal builtins set nt alone.  The MEMORY_EFFICIENT shape with the stores (20) or the loads (21) issued from inline
+// assembly with every combination of the three: POLICY bit 0 = sc0, bit 1 = sc1, bit 2 = nt.
+#define MB_POLICY_CASES(X) X(0, "") X(1, " sc0") X(2, " sc1") X(3, " sc0 sc1") X(4, " nt") X(5, " sc0 nt") X(6, " sc1 nt") X(7, " sc0 sc1 nt")
+template <int POLICY>
+__device__ __forceinline__ void st_policy(FS_GLOBAL f4* p, f4 v) {
+#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_store_dwordx4 %0, %1, off" BITS ::"v"(p), "v"(v) : "memory");
+    MB_POLICY_CASES(X)
+#undef X
+}
+template <int POLICY>
+__device__ __forceinline__ void st_policy(FS_GLOBAL f2* p, f2 v) {
+#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_store_dwordx2 %0, %1, off" BITS ::"v"(p), "v"(v) : "memory");
+    MB_POLICY_CASES(X)
+#undef X
+}
+template <int POLICY>
+__device__ __forceinline__ void ld_policy(f4& out, FS_GLOBAL const f4* p) {
+#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_load_dwordx4 %0, %1, off" BITS : "=v"(out) : "v"(p) : "memory");
+    MB_POLICY_CASES(X)
+#undef X
+}
+template <int POLICY>
+__device__ __forceinline__ void ld_policy(f2& out, FS_GLOBAL const f2* p) {
+#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_load_dwordx2 %0, %1, off" BITS : "=v"(out) : "v"(p) : "memory");
+    MB_POLICY_CASES(X)
+#undef X
+}
+template <int LOADS, int STORES>  // a policy, or -1 for the compiler's non-temporal builtin
+__global__ __launch_bounds__(64) void mb_memeff_both_policy(f2* p_, f4* m_, f4* v_, const f2* g_, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    f2 a, d;
+    f4 b, c;
+    if constexpr (LOADS < 0) {
+        a = ld<true>((FS_GLOBAL const f2*)p_ + i);
+        d = ld<true>((FS_GLOBAL const f2*)g_ + i);
+        b = ld<true>((FS_GLOBAL const f4*)m_ + i);
+        c = ld<true>((FS_GLOBAL const f4*)v_ + i);
+    } else {
+        ld_policy<LOADS>(a, (FS_GLOBAL const f2*)p_ + i);
+        ld_policy<LOADS>(d, (FS_GLOBAL const f2*)g_ + i);
+        ld_policy<LOADS>(b, (FS_GLOBAL const f4*)m_ + i);
+        ld_policy<LOADS>(c, (FS_GLOBAL const f4*)v_ + i);
+        // the compiler does not count loads it did not issue: wait for them here, with the values as operands so that
+        // nothing that uses them moves in front
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(d), "+v"(b), "+v"(c)::"memory");
+    }
+    const f4 g = {d[0], d[1], d[0], d[1]};
+    b = b * 0.9f + g * 0.1f;
+    c = c * 0.999f + g * g * 0.001f;
+    a[0] -= b[0] * 0.001f;
+    a[1] -= b[1] * 0.001f;
+    if constexpr (STORES < 0) {
+        st<true>((FS_GLOBAL f4*)m_ + i, b);
+        st<true>((FS_GLOBAL f4*)v_ + i, c);
+        st<true>((FS_GLOBAL f2*)p_ + i, a);
+    } else {
+        st_policy<STORES>((FS_GLOBAL f4*)m_ + i, b);
+        st_policy<STORES>((FS_GLOBAL f4*)v_ + i, c);
+        st_policy<STORES>((FS_GLOBAL f2*)p_ + i, a);
+    }
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
 __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -443,6 +508,22 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
             if (kind == 17) hipLaunchKernelGGL(mb_oneshot_phased, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq, period, split);
             else if (kind == 18) hipLaunchKernelGGL(mb_oneshot_x4_phased, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq, period, split);
             else hipLaunchKernelGGL(mb_memeff_both_phased, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq, period, split);
+            break;
+        }
+        case 20:
+        case 21:
+        case 22: {
+            // param: the policy bits (sc0 = 1, sc1 = 2, nt = 4) of the stores (20) or of the loads (21); the other side uses the builtin
+            if (param < 0 || param > 7) return -1;
+            const dim3 grid((uint32_t)grid64);
+#define X(N, BITS)                                                                                                                               \
+    if (param == N) {                                                                                                                            \
+        if (kind == 20) hipLaunchKernelGGL((mb_memeff_both_policy<-1, N>), grid, dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq);          \
+        else if (kind == 21) hipLaunchKernelGGL((mb_memeff_both_policy<N, -1>), grid, dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq);    \
+        else hipLaunchKernelGGL((mb_memeff_both_policy<N, 6>), grid, dim3(64), lds, stream, (f2*)p, M, V, (const f2*)g, nq);                      \
+    }
+            MB_POLICY_CASES(X)
+#undef X
             break;
         }
         default: return -1;
