@@ -665,7 +665,9 @@ int plan_zero_state(FsAdamPlan* plan, hipStream_t stream) {
     TableSlot& slot = plan->slots[plan->current];
     int rc = mark_order_after(slot.mark, stream);
     if (rc) return rc;
-    const size_t lds = 32768;  // a pass that only writes runs best with few waves per compute unit
+    // a pass that only writes through runs best with 10-13 waves per compute unit: 95-96 % of the HBM rate at 12-16 KiB of
+    // ballast, 85-90 % at 8 or 20 KiB, under 50 % from 32 KiB on (a wave's stores are acknowledged by the memory, not the L2)
+    const size_t lds = 14336;
     if (plan->mode == FSADAM_PURE_FP16)
         hipLaunchKernelGGL((fsadam_zero_state<FSADAM_PURE_FP16, kBlock>), dim3((uint32_t)n_blocks), dim3(kBlock), lds, stream, slot.d_table, tile_map(L));
     else

@@ -411,6 +411,97 @@ __global__ __launch_bounds__(64) void mb_memeff_both_policy(f2* p_, f4* m_, f4* 
     }
 }
 
+// 28: two streams of 16 bytes per lane written, 23: the write side of the MEMORY_EFFICIENT shape alone, 24: the 28-byte shape, 25: the 28-byte shape with four vectors per
+// lane (all loads, then all stores) -- each with the stores under policy STORES and the loads from the builtin.
+template <int STORES>
+__global__ __launch_bounds__(64) void mb_memeff_write_policy(f2* p_, f4* m_, f4* v_, int64_t n4, int pattern) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n4) return;
+    const f4 val = fill_value(i, pattern);
+    const f2 half = {val[0], val[1]};
+    st_policy<STORES>((FS_GLOBAL f4*)m_ + i, val);
+    st_policy<STORES>((FS_GLOBAL f4*)v_ + i, val);
+    st_policy<STORES>((FS_GLOBAL f2*)p_ + i, half);
+}
+template <int STORES>  // two streams of 16 bytes per lane: what zeroing fp16 or fp32 state writes
+__global__ __launch_bounds__(64) void mb_write2_policy(f4* m_, f4* v_, int64_t nq, int pattern) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    const f4 val = fill_value(i, pattern);
+    st_policy<STORES>((FS_GLOBAL f4*)m_ + i, val);
+    st_policy<STORES>((FS_GLOBAL f4*)v_ + i, val);
+}
+template <int STORES>
+__global__ __launch_bounds__(64) void mb_oneshot_policy(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + i;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + i;
+    f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+       d = ld<true>((FS_GLOBAL const f4*)g_ + i);
+    fake_update(a, b, c, d);
+    st_policy<STORES>(m, b);
+    st_policy<STORES>(v, c);
+    st_policy<STORES>(p, a);
+}
+template <int STORES>
+__global__ __launch_bounds__(64) void mb_oneshot_x4_policy(f4* p_, f4* m_, f4* v_, const f4* g_, int64_t nq) {
+    const int64_t base = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (base + 192 >= nq) return;
+    FS_GLOBAL f4* p = (FS_GLOBAL f4*)p_ + base;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)m_ + base;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)v_ + base;
+    FS_GLOBAL const f4* g = (FS_GLOBAL const f4*)g_ + base;
+    f4 a[4], b[4], c[4], d[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        a[k] = ld<true>((FS_GLOBAL const f4*)p + k * 64); b[k] = ld<true>((FS_GLOBAL const f4*)m + k * 64);
+        c[k] = ld<true>((FS_GLOBAL const f4*)v + k * 64); d[k] = ld<true>(g + k * 64);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fake_update(a[k], b[k], c[k], d[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st_policy<STORES>(m + k * 64, b[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st_policy<STORES>(v + k * 64, c[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) st_policy<STORES>(p + k * 64, a[k]);
+}
+
+// 26: the MEMORY_EFFICIENT shape with everything that can be varied around write-through stores: policy of the stores,
+// TILES consecutive tiles per wave (all loads, then all stores), BLOCK threads per workgroup (64, or 256 = four waves that
+// cover 4 KiB per fp32 stream between them), tiles in runs of 2^log2_run per XCD (0: dispatch order).
+template <int STORES, int TILES, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void mb_memeff_lab(f2* p_, f4* m_, f4* v_, const f2* g_, int64_t n4, int log2_run) {
+    const int64_t tile = log2_run ? xcd_tile(blockIdx.x, log2_run) : (int64_t)blockIdx.x;
+    const int64_t base = tile * (BLOCK * TILES) + threadIdx.x;
+    if (base + (TILES - 1) * BLOCK >= n4) return;  // the ragged end is left out
+    f2 a[TILES], d[TILES];
+    f4 b[TILES], c[TILES];
+#pragma unroll
+    for (int k = 0; k < TILES; ++k) {
+        a[k] = ld<true>((FS_GLOBAL const f2*)p_ + base + k * BLOCK);
+        d[k] = ld<true>((FS_GLOBAL const f2*)g_ + base + k * BLOCK);
+        b[k] = ld<true>((FS_GLOBAL const f4*)m_ + base + k * BLOCK);
+        c[k] = ld<true>((FS_GLOBAL const f4*)v_ + base + k * BLOCK);
+    }
+#pragma unroll
+    for (int k = 0; k < TILES; ++k) {
+        const f4 g = {d[k][0], d[k][1], d[k][0], d[k][1]};
+        b[k] = b[k] * 0.9f + g * 0.1f;
+        c[k] = c[k] * 0.999f + g * g * 0.001f;
+        a[k][0] -= b[k][0] * 0.001f;
+        a[k][1] -= b[k][1] * 0.001f;
+    }
+#pragma unroll
+    for (int k = 0; k < TILES; ++k) st_policy<STORES>((FS_GLOBAL f4*)m_ + base + k * BLOCK, b[k]);
+#pragma unroll
+    for (int k = 0; k < TILES; ++k) st_policy<STORES>((FS_GLOBAL f4*)v_ + base + k * BLOCK, c[k]);
+#pragma unroll
+    for (int k = 0; k < TILES; ++k) st_policy<STORES>((FS_GLOBAL f2*)p_ + base + k * BLOCK, a[k]);
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
 __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -524,6 +615,39 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
     }
             MB_POLICY_CASES(X)
 #undef X
+            break;
+        }
+        case 28:
+        case 23:
+        case 24:
+        case 25: {
+            if (param < 0 || param > 7) return -1;
+#define X(N, BITS)                                                                                                                               \
+    if (param == N) {                                                                                                                            \
+        if (kind == 28) hipLaunchKernelGGL(mb_write2_policy<N>, dim3((uint32_t)grid64), dim3(64), lds, stream, M, V, nq, g_pattern);                \
+        else if (kind == 23) hipLaunchKernelGGL(mb_memeff_write_policy<N>, dim3((uint32_t)grid64), dim3(64), lds, stream, (f2*)p, M, V, nq, g_pattern); \
+        else if (kind == 24) hipLaunchKernelGGL(mb_oneshot_policy<N>, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq);              \
+        else hipLaunchKernelGGL(mb_oneshot_x4_policy<N>, dim3((uint32_t)((nq + 255) / 256)), dim3(64), lds, stream, P, M, V, G, nq);               \
+    }
+            MB_POLICY_CASES(X)
+#undef X
+            break;
+        }
+        case 26: {
+            // param: bits 0-2 store policy (4 = nt, 6 = sc1 nt), bits 4-7 log2 of the run per XCD, bits 8-9 log2 of the tiles per
+            // wave (1, 2, 4), bit 12 workgroups of 256 threads
+            const int policy = param & 7, log2_run = (param >> 4) & 15, log2_tiles = (param >> 8) & 3, wide = (param >> 12) & 1;
+            if ((policy != 4 && policy != 6) || log2_tiles > 2) return -1;
+            const int64_t per_group = (wide ? 256 : 64) << log2_tiles;
+            int64_t grid = (nq + per_group - 1) / per_group;
+            if (log2_run) { const int64_t span = (int64_t)8 << log2_run; grid = (grid + span - 1) / span * span; }
+            if (grid > 0x7ffffff0) return -1;
+#define LAB(P, T, B)                                                                                                                    \
+    if (policy == P && (1 << log2_tiles) == T && (wide ? 256 : 64) == B)                                                                \
+        hipLaunchKernelGGL((mb_memeff_lab<P, T, B>), dim3((uint32_t)grid), dim3(B), lds, stream, (f2*)p, M, V, (const f2*)g, nq, log2_run);
+            LAB(4, 1, 64) LAB(4, 2, 64) LAB(4, 4, 64) LAB(4, 1, 256) LAB(4, 2, 256) LAB(4, 4, 256)
+            LAB(6, 1, 64) LAB(6, 2, 64) LAB(6, 4, 64) LAB(6, 1, 256) LAB(6, 2, 256) LAB(6, 4, 256)
+#undef LAB
             break;
         }
         default: return -1;
