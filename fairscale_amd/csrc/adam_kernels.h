@@ -25,7 +25,7 @@ struct VecOf {
     typedef type in_memory __attribute__((aligned(sizeof(T))));
 };
 
-// E consecutive elements of one stream, one instruction, non-temporal.
+// E consecutive elements of one stream, one instruction: loads non-temporal, stores written through.
 template <typename T, int E>
 __device__ __forceinline__ typename VecOf<T, E>::type load_vec(gptr<const T> ptr) {
     using V = typename VecOf<T, E>::in_memory;

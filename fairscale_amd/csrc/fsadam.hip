@@ -12,13 +12,14 @@
 //   * every workgroup is "one-shot": it handles one small tile (a few KiB per stream) and exits, so
 //     that the hardware dispatcher hands out tiles in address order and the set of DRAM pages in
 //     use at any moment stays small (grid-stride loops let workgroups drift apart and lose ~20 %);
-//   * only 6-12 waves are resident per compute unit: enough bytes in flight to cover the latency,
+//   * only 10-13 waves are resident per compute unit: enough bytes in flight to cover the latency,
 //     few enough that the active address window stays tight.  Residency is capped by giving each
 //     workgroup a block of LDS it never touches (LDS is the one launch-time resource that bounds
 //     residency without costing registers or bandwidth);
 //   * every load/store instruction of a wave covers one contiguous span (lane i next to lane i+1),
-//     128 bits per lane for fp32 streams and 64 or 128 bits per lane for fp16 streams, all with
-//     the non-temporal hint (nothing is re-read).
+//     128 bits per lane for fp32 streams and 64 or 128 bits per lane for fp16 streams; loads carry
+//     the non-temporal hint (nothing is re-read) and stores are written through the L2 at device
+//     scope on top of it (store_through in fsadam_common.h: 2 points of the HBM rate).
 // The tensor list becomes a device-resident table of 64-byte chunk descriptors (five pointers
 // already advanced to the chunk, element count), uploaded once and reused every step.  Consecutive
 // tensors that continue each other in every stream are laid out as one (build_runs).  A wave finds its work with one shift and one scalar load: descriptor = table[block >> k],
