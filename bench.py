@@ -556,6 +556,7 @@ def run_micro(torch, args, device):
     measure("reads and writes (22 B/element), stores [sc1 nt], four tiles per wave, ballast 40960 B", 26, 22, lds=40960, param=lab(tiles=2))
     measure("reads and writes (22 B/element), stores [sc1 nt], workgroups of 256 threads, ballast 32768 B", 26, 22, lds=32768, param=lab(wide=1))
     measure("reads and writes (22 B/element), stores [sc1 nt], runs of 4 tiles per XCD, ballast 10240 B", 26, 22, lds=10240, param=lab(run=2))
+    measure("reads and writes (22 B/element), stores [sc1 nt], half a tile per wave (8 and 4 bytes per lane), ballast 7168 B", 29, 22, lds=7168)
     by = {r["variant"]: r for r in results}
     r_gbs = by["reads only (12 B/element), ballast 12288 B"]["gbs_at_median"]
     w_gbs = by["writes only (10 B/element), ballast 12288 B"]["gbs_at_median"]

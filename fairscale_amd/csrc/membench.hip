@@ -502,6 +502,23 @@ __global__ __launch_bounds__(BLOCK) void mb_memeff_lab(f2* p_, f4* m_, f4* v_, c
     for (int k = 0; k < TILES; ++k) st_policy<STORES>((FS_GLOBAL f2*)p_ + base + k * BLOCK, a[k]);
 }
 
+// 29: the MEMORY_EFFICIENT shape with half the bytes per wave: 8 bytes per lane of the fp32 streams, 4 of the fp16 ones
+// (128 elements per wave instead of 256), stores written through.
+__global__ __launch_bounds__(64) void mb_memeff_half_tile(float* p_, f2* m_, f2* v_, const float* g_, int64_t n2) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i >= n2) return;
+    float a = ld<true>((FS_GLOBAL const float*)p_ + i);          // two halves
+    const float d = ld<true>((FS_GLOBAL const float*)g_ + i);    // two halves
+    f2 b = ld<true>((FS_GLOBAL const f2*)m_ + i), c = ld<true>((FS_GLOBAL const f2*)v_ + i);
+    const f2 g = {d, d};
+    b = b * 0.9f + g * 0.1f;
+    c = c * 0.999f + g * g * 0.001f;
+    a -= b[0] * 0.001f;
+    asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"((FS_GLOBAL f2*)m_ + i), "v"(b) : "memory");
+    asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"((FS_GLOBAL f2*)v_ + i), "v"(c) : "memory");
+    asm volatile("global_store_dword %0, %1, off sc1 nt" ::"v"((FS_GLOBAL float*)p_ + i), "v"(a) : "memory");
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
 __global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
@@ -631,6 +648,12 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
     }
             MB_POLICY_CASES(X)
 #undef X
+            break;
+        }
+        case 29: {
+            const int64_t n2 = numel / 2, grid = (n2 + 63) / 64;
+            if (grid > 0x7ffffff0) return -1;
+            hipLaunchKernelGGL(mb_memeff_half_tile, dim3((uint32_t)grid), dim3(64), lds, stream, (float*)p, (f2*)m, (f2*)v, (const float*)g, n2);
             break;
         }
         case 26: {
