@@ -805,7 +805,7 @@ void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* waves, int64
     // a pass that only reads pays for every small store it makes: 16 tiles share one partial
     *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
-    *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 13312 : 16384);
+    *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 12288 : 16384);  // writes: written through, plateau 11-12.5 KiB
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
@@ -1294,7 +1294,7 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
     // vectors per lane and ballast as fsadam_grad_pass chooses them.  Options are not consulted.
     const bool writes = write_back != 0 && !(inv_scale_dev == nullptr && inv_scale == 1.0f);
     const int64_t waves = 16, items = writes ? 4 : 8;
-    const size_t lds = writes ? 13312 : 16384;
+    const size_t lds = writes ? 12288 : 16384;
     const Layout L = grad_layout(grads, n_tensors, grad_dtype, items, /*align_heads=*/1, /*mid_tiles=*/16);
     const int64_t n_descs = L.descs(), n_groups = ceil_div(L.blocks(), waves);
     if (n_descs > FSADAM_NOALLOC_MAX_DESCRIPTORS)

@@ -131,7 +131,7 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint
                 else raw[k][e] = __builtin_bit_cast(uint32_t, grad_float<HOW>(__builtin_bit_cast(float, word), inv_scale, acc));
             }
             if (WRITE && HOW != kGradUnit)
-                __builtin_nontemporal_store(raw[k], reinterpret_cast<gptr<u32x4_in_memory>>(g + (k * BLOCK + lane) * E));
+                store_through((gptr<void>)(g + (k * BLOCK + lane) * E), raw[k]);
         }
     } else {
         for (uint32_t e = lane; e < left; e += BLOCK) {

@@ -134,7 +134,7 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   running on the caller's stream; 0: the copy is enqueued on the caller's stream
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
  *                   4 for one that writes the gradients back (default 0)
- *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 13312 likewise
+ *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 12288 likewise
  *   "grad_waves"    gradient pass: tiles (one wave each) per workgroup, 1, 4 or 16; the workgroup writes one
  *                   partial result.  0 = 16 for a read-only pass, 1 for one that writes back (default 0)
  * A workgroup of the step is one wave64 handling one vector per lane and stream, tiles are taken in dispatch order
