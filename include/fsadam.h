@@ -116,7 +116,7 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
 /* Tuning knobs, by name; returns FSADAM_EINVAL for an unknown name or a value out of range.
  *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
  *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
- *                   per-mode default (12-16 KiB, default)
+ *                   per-mode default (12-15 KiB, default)
  *   "merge_runs"    1 (default): consecutive rows of a list that continue each other in every stream (p, m, v, g and
  *                   the fp16 copy each start where the row before ended: parameters that are back-to-back views of
  *                   one buffer, with gradients and state laid out alike) are laid out as ONE tensor, so that a
