@@ -533,3 +533,22 @@ def test_versioned_state_map_counts_what_changes_the_key_set():
     st["x"]["step"] = 7
     for clone in (pickle.loads(pickle.dumps(st)), copy.deepcopy(st)):
         assert type(clone) is _VersionedState and clone["x"] == {"step": 7} and clone["fresh"] == {}
+
+
+def test_wide_assembly_stores_carry_their_wait_states():
+    """The write-through store comes from inline assembly, so the compiler does not keep vector instructions away from the
+    store's data registers for the two wait states a store of more than 64 bits needs on gfx950: the assembly text has to.
+    (What happens without them: a parameter per lane comes out wrong in FULL_PRECISION with fp16 copies, which the GPU suite
+    shows.)  Every 128-bit store in an asm statement of the library's sources is followed by `s_nop 1` in the same statement."""
+    import glob
+    import re
+
+    src_dir = os.path.join(REPO, "fairscale_amd", "csrc")
+    wide = 0
+    for path in glob.glob(os.path.join(src_dir, "fsadam*.h")) + glob.glob(os.path.join(src_dir, "*_kernels.h")) + [os.path.join(src_dir, "fsadam.hip")]:
+        text = open(path).read()
+        for statement in re.findall(r'asm volatile\((.*?)\);', text, flags=re.S):
+            if "global_store_dwordx4" in statement or "global_store_dwordx3" in statement:
+                wide += 1
+                assert re.search(r'global_store_dwordx[34][^"]*\\n\\ts_nop 1"', statement), f"{path}: a wide store without its wait states"
+    assert wide >= 1
