@@ -58,11 +58,12 @@
 // The descriptor table and the partial results of a gradient pass for callers that cannot allocate: one
 // array per GPU, part of the loaded code object, held until the process ends.  Layout: the table
 // (FSADAM_NOALLOC_MAX_DESCRIPTORS rows of 64 bytes), then the partials of the tiles' workgroups
-// (FSADAM_NOALLOC_MAX_WORKGROUPS), of the second reduction stage (512) and the total (1), 16 bytes each.
+// (FSADAM_NOALLOC_MAX_WORKGROUPS, and 7 more because the slots are handed out in eights), of the second reduction
+// stage (512) and the total (1), 16 bytes each.
 // In host code the name below is only a handle for hipGetSymbolAddress: the device address is looked up
 // once per device (scratch_on_current_device) and only that pointer is ever handed to a kernel.
 constexpr size_t kScratchTableBytes = (size_t)FSADAM_NOALLOC_MAX_DESCRIPTORS * 64;
-constexpr size_t kScratchPartials = (size_t)FSADAM_NOALLOC_MAX_WORKGROUPS + 512 + 1;
+constexpr size_t kScratchPartials = (size_t)FSADAM_NOALLOC_MAX_WORKGROUPS + 7 + 512 + 1;  // 7: the slots are handed out in eights
 constexpr size_t kScratchBytes = kScratchTableBytes + kScratchPartials * 16;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
@@ -99,14 +100,16 @@ struct Options {
 };
 
 // Residency that measured fastest with one wave64 per workgroup, one vector per lane per stream and stores that
-// are written through (store_through): about 40 KiB of loads in flight per compute unit, i.e. 10 waves of the
-// 4 KiB-per-wave modes and 13 of the 2-3 KiB-per-wave ones (160 KiB of LDS / ballast = resident workgroups).
-// Each value is the middle of a plateau about 1 KiB wide either way; 2 KiB off costs 2-8 points.
+// are written through (store_through): about 36 KiB of loads in flight per compute unit, i.e. 9 waves of the
+// 4 KiB-per-wave modes and 12 of the 3 KiB-per-wave ones.  The hardware hands out LDS in granules of 1280 bytes
+// (a sweep in steps of 256 bytes changes the rate only at multiples of 1280), so a ballast of B bytes allows
+// floor(128 / ceil(B / 1280)) workgroups per compute unit: 12 288 -> 12, 14 080 -> 11, 15 360 -> 10, 16 640 and
+// 17 920 -> 9, 19 200 -> 8; 13 and 15 cannot be had.  One wave more or less costs 0.3-1.5 points, two cost 2-4.
 int64_t default_lds_throttle(int mode) {
     switch (mode) {
-        case FSADAM_FULL_PRECISION: return 15360;
-        case FSADAM_FULL_PRECISION_FP16_COPY: return 15360;
-        case FSADAM_MIXED_PRECISION: return 15360;
+        case FSADAM_FULL_PRECISION: return 16640;
+        case FSADAM_FULL_PRECISION_FP16_COPY: return 16640;
+        case FSADAM_MIXED_PRECISION: return 16640;
         case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
         default: return 12288;
     }
@@ -701,6 +704,7 @@ struct GradPlan {
 };
 
 constexpr int kReduceBlocks = 512;
+constexpr int kSlotSlack = 7;  // the partials of n workgroups take 8 * ceil(n / 8) slots
 
 int grad_elem_size(int dtype) { return dtype == FSADAM_GRAD_F16 ? 2 : 4; }
 int64_t grad_tile_elems(int dtype, int64_t items) { return 64 * (16 / grad_elem_size(dtype)) * items; }
@@ -795,17 +799,17 @@ void grad_plan_free(GradPlan* plan) {
     delete plan;
 }
 
-// Measured best shapes: a read-only pass wants more bytes per wave (8 vectors, 16 KiB ballast);
-// a pass that also writes the gradients back behaves like the Adam kernels (4 vectors, 13 KiB).
+// Measured best shapes, one wave per workgroup either way (consecutive tiles then run on different XCDs, which
+// the memory channels like best): a pass that only reads takes 8 vectors per lane (8 KiB per wave) at 11 waves per
+// compute unit, a pass that writes the gradients back 4 vectors at 12 waves, like the Adam kernels.
 void grad_shape(bool writes, int64_t* items, int64_t* lds, int64_t* waves, int64_t* align_heads, int64_t* mid_tiles, int64_t* upload_stream) {
     std::lock_guard<std::mutex> lock(g_mutex);
     *upload_stream = g_opt.upload_stream;
     *mid_tiles = g_opt.mid_tiles;
     *align_heads = g_opt.align_heads;
-    // a pass that only reads pays for every small store it makes: 16 tiles share one partial
-    *waves = g_opt.grad_waves ? g_opt.grad_waves : (writes ? 1 : 16);
+    *waves = g_opt.grad_waves ? g_opt.grad_waves : 1;
     *items = g_opt.grad_items ? g_opt.grad_items : (writes ? 4 : 8);
-    *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 12288 : 16384);  // writes: written through, plateau 11-12.5 KiB
+    *lds = g_opt.grad_lds_throttle >= 0 ? g_opt.grad_lds_throttle : (writes ? 12800 : 14080);
 }
 
 int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStream_t stream) {
@@ -834,14 +838,14 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
         }
         slot.cap_descs = cap;
     }
-    if (n_blocks + kReduceBlocks + 1 > plan->cap_partials) {
+    if (n_blocks + kSlotSlack + kReduceBlocks + 1 > plan->cap_partials) {
         // the partials may still be read by the reduction of the previous call
         rc = mark_wait(plan->partials_mark);
         if (rc) return rc;
         if (plan->d_partials) (void)hipFree(plan->d_partials);
         plan->d_partials = nullptr;
         plan->cap_partials = 0;
-        const int64_t cap = n_blocks + n_blocks / 8 + kReduceBlocks + 1;
+        const int64_t cap = n_blocks + kSlotSlack + n_blocks / 8 + kReduceBlocks + 1;
         if (hipMalloc(reinterpret_cast<void**>(&plan->d_partials), cap * sizeof(GradPartial)) != hipSuccess) {
             plan->d_partials = nullptr;
             return fail(FSADAM_ENOMEM, "hipMalloc of the partial sums failed");
@@ -874,9 +878,12 @@ int grad_launch(const ChunkDesc* table, const Layout& L, int64_t waves, int64_t 
     const int64_t n_blocks = L.blocks();
     const TileMap map = tile_map(L);
     const int64_t n_groups = ceil_div(n_blocks, waves);
+    // the workgroups' partials lie in 8 rows of per_xcd slots (see fsadam_grad_tiles): n_slots <= n_groups + kSlotSlack
+    const uint32_t per_xcd = (uint32_t)ceil_div(std::max<int64_t>(n_groups, 1), 8);
+    const int64_t n_slots = (int64_t)per_xcd * 8;
 #define FS_GRAD_LAUNCH(WAVES, ITEMS)                                                                                          \
     hipLaunchKernelGGL((fsadam_grad_tiles<T, WAVES, ITEMS>), dim3((uint32_t)n_groups), dim3(64 * WAVES), lds, stream,        \
-                       table, map, (uint32_t)n_blocks, inv_scale, inv_scale_dev, write_back, first)
+                       table, map, (uint32_t)n_blocks, inv_scale, inv_scale_dev, write_back, first, per_xcd)
 #define FS_GRAD_ITEMS(WAVES)                          \
     do {                                              \
         if (items == 2) FS_GRAD_LAUNCH(WAVES, 2);      \
@@ -892,12 +899,12 @@ int grad_launch(const ChunkDesc* table, const Layout& L, int64_t waves, int64_t 
 #undef FS_GRAD_LAUNCH
     FS_HIP(hipGetLastError());
     // two fixed-shape reduction steps, the second of which publishes (also when the list holds no element: everything is zero)
-    const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_groups, 1024)));
-    const uint32_t per_block = (uint32_t)ceil_div(std::max<int64_t>(n_groups, 1), blocks2);
-    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_groups, per_block, second, 0, 0,
-                       (float*)nullptr, (double*)nullptr, (float*)nullptr);
+    const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_slots, 1024)));
+    const uint32_t per_block = (uint32_t)ceil_div(n_slots, blocks2);
+    hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_slots, per_block, second, 0, 0,
+                       (float*)nullptr, (double*)nullptr, (float*)nullptr, per_xcd, (uint32_t)n_groups);
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total, 1, (int)(sizeof(T) == 2),
-                       found_inf, sum_squares, abs_max);
+                       found_inf, sum_squares, abs_max, 0u, 0u);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
@@ -1308,7 +1315,7 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
     if (int rc = scratch_on_current_device(&base)) return rc;
     ChunkDesc* table = reinterpret_cast<ChunkDesc*>(base);
     GradPartial* first = reinterpret_cast<GradPartial*>(base + kScratchTableBytes);
-    GradPartial* second = first + FSADAM_NOALLOC_MAX_WORKGROUPS;
+    GradPartial* second = first + FSADAM_NOALLOC_MAX_WORKGROUPS + kSlotSlack;
     GradPartial* total = second + kReduceBlocks;
     if (!grad_fill_table(g_scratch_staging, L, grads, n_tensors, grad_elem_size(grad_dtype), 1))
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");

@@ -142,15 +142,20 @@ __device__ __forceinline__ void grad_tile(const ChunkDesc& d, uint32_t off, uint
 }
 
 // One wave = one tile of 64 x ITEMS 16-byte vectors, found through the table like the tiles of the
-// Adam step.  A workgroup is WAVES consecutive tiles and writes ONE partial: in a pass that only
-// reads, every small store forces a read/write turnaround somewhere in the DRAM, and one 16-byte
-// store per wave (400 000 of them over the benchmark's shard) was measured to cost 5-8 % of the read
-// bandwidth; with 16 waves per workgroup the cost is gone.  `n_tiles`: tiles really there (the last
-// workgroup may have fewer than WAVES).
+// Adam step.  A workgroup is WAVES consecutive tiles and writes ONE partial of 16 bytes.  Those small
+// stores are what a pass over the gradients pays for besides its stream: written through one by one
+// (400 000 to 800 000 stores of a quarter of a 64-byte memory word each) they cost a pass that only reads
+// 5-8 % and a pass that writes back 2.5 %.  They are therefore ordinary cached stores, and workgroup b
+// writes slot (b mod 8) * per_xcd + b / 8: the hardware deals consecutive workgroups out to the eight XCDs
+// in turn, each XCD has an L2 of its own, so the eight partials that make up one 128-byte line all come
+// from the same L2, a few workgroups apart in time, and leave it as one full line.  (Nothing depends on
+// which XCD a workgroup really runs on: the slot is a function of the workgroup's number alone, and the
+// reduction reads the slots in a fixed order.)  `n_tiles`: tiles really there (the last workgroup may
+// have fewer than WAVES); `per_xcd`: ceil(workgroups / 8).
 template <typename T, int WAVES, int ITEMS>
 __global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc* __restrict__ table, TileMap map, uint32_t n_tiles, float inv_scale_value,
                                                                 const float* __restrict__ inv_scale_dev, int write_back,
-                                                                GradPartial* __restrict__ partials) {
+                                                                GradPartial* __restrict__ partials, uint32_t per_xcd) {
     constexpr int BLOCK = 64;
     constexpr uint32_t kTile = BLOCK * GradTraits<T>::kElems * ITEMS;
     // the wave's number within the workgroup is the same for all its lanes: say so, and the tile's
@@ -224,21 +229,26 @@ __global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc*
             }
         }
     }
-    if (threadIdx.x == 0) {  // the 16 bytes in one store that is written through: 1.5 points of a pass that only reads
+    if (threadIdx.x == 0) {
         GradPartial part;
         part.sum_squares = dsum;
         part.stored_max = smax;
         part.incoming_max = imax;
-        store_through((gptr<void>)(partials + blockIdx.x), part);
+        // one ordinary (cached) 16-byte store
+        *((gptr<grad_words_t>)reinterpret_cast<grad_words_t*>(partials) + ((blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3))) =
+            __builtin_bit_cast(grad_words_t, part);
     }
 }
 
 // Fixed-order reduction of `n` partials into `out[blockIdx.x]`: block b takes the b-th contiguous
-// slice, thread t every 256th entry of it, then a shared-memory tree.  The last step (one block,
+// slice, thread t every 256th entry of it, then a shared-memory tree.  `per_xcd` != 0: `in` holds the
+// partials of `n_groups` workgroups in the slots fsadam_grad_tiles chose (8 rows of per_xcd slots, n = 8 * per_xcd);
+// the slots at the end of a row that belong to no workgroup are skipped.  The last step (one block,
 // `publish` set) hands the result to the caller's three outputs instead.
 __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
                                                           GradPartial* __restrict__ out, int publish, int is_half,
-                                                          float* found_inf, double* sum_squares, float* abs_max) {
+                                                          float* found_inf, double* sum_squares, float* abs_max,
+                                                          uint32_t per_xcd, uint32_t n_groups) {
     __shared__ double s_sum[256];
     __shared__ uint32_t s_stored[256];
     __shared__ uint32_t s_incoming[256];
@@ -247,6 +257,10 @@ __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __r
     double sum = 0.0;
     uint32_t stored = 0, incoming = 0;
     for (uint32_t i = lo + threadIdx.x; i < hi; i += 256) {
+        if (per_xcd) {  // slot i = row * per_xcd + column belongs to workgroup column * 8 + row
+            const uint32_t row = i / per_xcd, column = i - row * per_xcd;
+            if (column * 8u + row >= n_groups) continue;
+        }
         const GradPartial p = in[i];
         sum += p.sum_squares;
         stored = p.stored_max > stored ? p.stored_max : stored;

@@ -253,12 +253,12 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
 /* fsadam_grad_pass for callers that cannot allocate device memory: code that runs between the begin and end of
  * a HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference
  * (its gradient passes are torch operators, which allocate their outputs).  Same arguments, same results:
- * what is stored, the flag and the maximum have the bits fsadam_grad_pass gives; the sum of squares is
- * bit-identical for a pass that writes nothing back and within 1e-6 relative otherwise (16 tiles always share one
- * partial here).  The call makes no hipMalloc / hipFree / hipHostMalloc, creates no stream or event and copies
+ * what is stored, the flag and the maximum have the bits fsadam_grad_pass gives; the sum of squares agrees
+ * within 1e-6 relative (16 tiles share one partial here, each tile has its own there, so the additions group
+ * differently).  The call makes no hipMalloc / hipFree / hipHostMalloc, creates no stream or event and copies
  * nothing with the copy engines: the descriptor table travels in kernel arguments (one small launch per 48
  * rows) and lives, with the partial results, in an array that is part of the library's code object,
- * FSADAM_NOALLOC_MAX_DESCRIPTORS * 64 + (FSADAM_NOALLOC_MAX_WORKGROUPS + 513) * 16 bytes (1.26 MiB) per GPU,
+ * FSADAM_NOALLOC_MAX_DESCRIPTORS * 64 + (FSADAM_NOALLOC_MAX_WORKGROUPS + 520) * 16 bytes (1.26 MiB) per GPU,
  * held until the process ends.  A list that needs more descriptors or workgroups than that is refused with
  * FSADAM_EINVAL (a workgroup covers 65536 fp16 / 32768 fp32 elements when the pass only reads, half as many
  * when it writes back: at least 1.07e9 elements in every case; a tensor of 131072 elements or more takes one
