@@ -55,9 +55,9 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-numel", type=int, default=1 << 26, help="sample size of the CPU baseline")
     ap.add_argument("--calib-copy-bytes", type=int, default=0,
-                    help="first run the library's plain copy kernel over this many bytes three times (a dispatch of known "
-                         "traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--micro", action="store_true", help="run the structure microbenchmarks instead (needs libfsadam_membench.so) and print a table")
+                    help="first run the microbenchmark library's plain copy kernel over this many bytes three times (a dispatch of "
+                         "known traffic, for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--micro", action="store_true", help="run the structure microbenchmarks instead (libfsadam_membench.so, built on demand) and print a table")
     ap.add_argument("--micro-numel", type=int, default=SHARD_NUMEL)
     ap.add_argument("--micro-data", default="random", choices=["random", "zeros"],
                     help="what the microbenchmark's buffers hold and its write-only kernels store (the bandwidth of this part depends on it)")
@@ -236,14 +236,16 @@ def measure_grad_pass(torch, numel, steps, warmup, device):
         for _ in range(warmup):
             grad_pass([g], inv, write_back=write_back)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        events[0].record()
+        for i in range(steps):
             grad_pass([g], inv, write_back=write_back)
-        e1.record()
+            events[i + 1].record()
         torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / steps
-        out[name] = {"ms": ms, "bytes_per_param": bpp, "achieved_gbs": numel * bpp / ms / 1e6, "frac_of_hbm_peak": numel * bpp / ms / 1e6 / HBM_PEAK_GBS}
+        ms = events[0].elapsed_time(events[steps]) / steps
+        median = spread([events[i].elapsed_time(events[i + 1]) for i in range(steps)])["median"]
+        out[name] = {"ms": ms, "ms_median": median, "bytes_per_param": bpp, "achieved_gbs": numel * bpp / ms / 1e6,
+                     "frac_of_hbm_peak": numel * bpp / ms / 1e6 / HBM_PEAK_GBS, "frac_at_median": numel * bpp / median / 1e6 / HBM_PEAK_GBS}
     del g
     torch.cuda.empty_cache()
     return out
@@ -445,6 +447,19 @@ def load_traffic(workload_key):
     return int(found.group(1)) if found else None
 
 
+def load_membench():
+    """The microbenchmark library (fairscale_amd/csrc/membench.hip), compiled first when it is missing or older than its
+    source: nothing in the product loads it, so the ordinary build leaves it out."""
+    import ctypes
+
+    from fairscale_amd.csrc import build as csrc_build
+
+    if not csrc_build.membench_is_current():
+        print(f"building {csrc_build.MEMBENCH_LIBRARY} ...", file=sys.stderr, flush=True)
+        csrc_build.build_membench()
+    return ctypes.CDLL(csrc_build.MEMBENCH_LIBRARY)
+
+
 def run_micro(torch, args, device):
     """The measurements the kernel's shape rests on, from kernels the tree builds (fairscale_amd/csrc/membench.hip):
     one-shot tiles against a grid-stride loop, residency (LDS ballast) sweep, temporal against non-temporal accesses,
@@ -453,11 +468,7 @@ def run_micro(torch, args, device):
     writes only and the step's mix.  Prints one line per variant and one JSON line at the end."""
     import ctypes
 
-    path = os.path.join(REPO, "fairscale_amd", "csrc", "libfsadam_membench.so")
-    if not os.path.exists(path):
-        print(f"{path} is missing: build it with `python -m fairscale_amd.csrc.build`", file=sys.stderr)
-        sys.exit(1)
-    L = ctypes.CDLL(path)
+    L = load_membench()
     vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
     L.fsadam_membench_launch.restype = i32
     L.fsadam_membench_launch.argtypes = [i32, vp, vp, vp, vp, i64, i32, i32, vp, vp, vp]
@@ -511,6 +522,15 @@ def run_micro(torch, args, device):
     measure("table of descriptors, ONE scalar load per wave, ballast 16384 B", 4, 28, lds=16384)
     measure("table of descriptors staged in LDS + barrier, ballast 16384 B (incl. the 64 B staged)", 3, 28, lds=16384 - 64)
     measure("table of descriptors staged in LDS + barrier, no ballast", 3, 28)
+    print("# the same two ways to the descriptor with the stores written through (sc1 nt), each over its own range of ballasts")
+    for lds in (8960, 11520, 14080, 16640, 19200):
+        measure(f"28 B shape, table, ONE scalar load per wave, stores [sc1 nt], ballast {lds:5d} B", 30, 28, lds=lds)
+        measure(f"28 B shape, table staged in LDS + barrier, stores [sc1 nt], ballast {lds:5d} B (incl. the 64 B staged)", 31, 28, lds=lds - 64)
+    launch(-2)  # the table again, for p and g as fp16 streams
+    for lds in (6400, 8960, 10240, 11520, 12800, 14080):
+        measure(f"22 B shape, table, ONE scalar load per wave, stores [sc1 nt], ballast {lds:5d} B", 32, 22, lds=lds)
+        measure(f"22 B shape, table staged in LDS + barrier, stores [sc1 nt], ballast {lds:5d} B (incl. the 64 B staged)", 33, 22, lds=lds - 64)
+    launch(-1)
     measure("reads only, four fp32 streams (16 B/element), ballast 16384 B", 5, 16, lds=16384)
     measure("writes only, three fp32 streams (12 B/element), ballast 16384 B", 6, 12, lds=16384)
     print("# the write side on its own (fp32 streams)")
@@ -594,11 +614,17 @@ def main():
         run_micro(torch, args, device)
         return
     if args.calib_copy_bytes > 0:
+        import ctypes
+
+        M = load_membench()
+        M.fsadam_membench_copy.restype = ctypes.c_int
+        M.fsadam_membench_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         n = args.calib_copy_bytes // 16 * 16
         src = torch.zeros(n, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
         for _ in range(3):
-            _cabi.check(_cabi.lib().fsadam_calib_copy(dst.data_ptr(), src.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+            rc = M.fsadam_membench_copy(dst.data_ptr(), src.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, f"fsadam_membench_copy returned {rc}"
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
@@ -630,6 +656,27 @@ def main():
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"
+    # every measured configuration in a few numbers each, under a key of its own next to the headline's roofline:
+    # ms per step (kernel time for the flat shard, device time per step for the lists), the fraction of the HBM peak that
+    # gives over the run, and the fraction at the median step
+    frac_of = lambda numel, bpp, ms: numel * bpp / ms / 1e6 / HBM_PEAK_GBS  # noqa: E731
+    configs = {workload: {"ms": main_res["kernel_ms"], "frac": frac_of(args.numel, main_res["bytes_per_param"], main_res["kernel_ms"]),
+                          "frac_at_median": frac_of(args.numel, main_res["bytes_per_param"], main_res["kernel_ms_median"])}}
+    for key, r in also.items():
+        if key in BYTES_PER_PARAM:
+            configs[f"flat_shard_{args.numel}_{key}"] = {"ms": r["kernel_ms"], "frac": r["frac_of_hbm_peak"],
+                                                         "frac_at_median": frac_of(args.numel, r["bytes_per_param"], r["kernel_ms_median"])}
+        elif key == "grad_pass_fp16":
+            for name, g in r.items():
+                configs[f"grad_pass_fp16_{name}_{args.numel}"] = {"ms": g["ms"], "frac": g["frac_of_hbm_peak"], "frac_at_median": g["frac_at_median"]}
+        elif key.startswith("c1_"):
+            configs[key] = {"ms": r["gpu"]["device_ms_median"], "frac": None, "frac_at_median": None,
+                            "cpu_ms": r["cpu"]["ms_per_step"], "note": "cache-resident: no HBM statement"}
+        elif "skipped" not in r:
+            configs[key] = {"ms": r["ms_per_step"], "frac": r["frac_of_hbm_peak"], "frac_at_median": r["frac_of_hbm_peak_at_median"]}
+            if "overflow_step" in r:
+                configs[key]["overflow_step_ms"] = r["overflow_step"]["ms"]
+                configs[key]["clean_step_after_backoff_ms"] = r["clean_step_after_backoff_ms"]
     # the committed counter summary speaks for default options only
     traffic = load_traffic(workload) if not args.opt else None
     traffic_source = (f"profiles/{TRAFFIC_SUMMARIES[workload]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload at default options; "
@@ -658,7 +705,7 @@ def main():
                      "kernel_ms_min": main_res["kernel_ms_min"],
                      "kernel_ms_median": main_res["kernel_ms_median"], "kernel_ms_max": main_res["kernel_ms_max"],
                      "frac_at_median": args.numel * main_res["bytes_per_param"] / main_res["kernel_ms_median"] / 1e6 / HBM_PEAK_GBS,
-                     "bytes_per_param": main_res["bytes_per_param"]},
+                     "bytes_per_param": main_res["bytes_per_param"], "configs": configs},
         "cpu_baseline": cpu,
         "also": also,
     }

@@ -19,8 +19,7 @@ FULL_PRECISION_FP16_COPY = 4
 
 ABI_VERSION = 3
 
-# $FSADAM_LIBRARY names another build of the same ABI (the measurement variants of csrc/build.py); normally unset
-_LIB_PATH = os.environ.get("FSADAM_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
 
 
 class FsAdamTensor(ctypes.Structure):
@@ -88,7 +87,6 @@ SIGNATURES = {
     "fsadam_grad_pass": (_i32, [ctypes.POINTER(FsGradTensor), _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _vp]),
     "fsadam_grad_pass_noalloc": (_i32, [ctypes.POINTER(FsGradTensor), _i64, _i32, _f32, _vp, _i32, _vp, _vp, _vp, _vp]),
     "fsadam_clear_cache": (_i32, []),
-    "fsadam_calib_copy": (_i32, [_vp, _vp, _i64, _vp]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

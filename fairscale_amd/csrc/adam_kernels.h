@@ -87,17 +87,8 @@ __device__ __forceinline__ void adam_update(const StepScalars& s, float in_p, fl
         out_m = momentum;
         out_v = velocity;
     }
-#ifdef FSADAM_EXPERIMENT_APPROX_DIV_SQRT
-    // Measurement aid, never defined for the library that ships (csrc/build.py --experiment-approx builds a second
-    // library with it): the hardware's approximate square root and reciprocal (1 ulp) instead of the correctly rounded
-    // ones, which takes about 20 of the 53 vector operations per element out of PURE_FP16.  It was built to find out
-    // whether that mode is bound by the vector units; the step got 0.7 % faster, so it is not.
-    const float denom = (EPS_MODE == 0) ? __builtin_amdgcn_sqrtf(velocity + s.eps) : __builtin_amdgcn_sqrtf(velocity) + s.eps;
-    const float update = momentum * __builtin_amdgcn_rcpf(denom) + s.decay * in_p;
-#else
     const float denom = (EPS_MODE == 0) ? sqrtf(velocity + s.eps) : sqrtf(velocity) + s.eps;
     const float update = momentum / denom + s.decay * in_p;
-#endif
     out_p = as_float32(in_p - s.step_size * update);
 }
 

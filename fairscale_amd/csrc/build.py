@@ -1,7 +1,8 @@
 """Compiles fsadam.hip (with the kernel headers next to it) into libfsadam.so next to this file (hipcc, gfx950 only), and the host-side
 helper tensor_rows.cpp into a CPython extension module (g++, against the installed torch).
 
-Usage: ``python -m fairscale_amd.csrc.build``, or ``build_library()`` / ``build_rows_module()``.  Both
+Usage: ``python -m fairscale_amd.csrc.build`` (``--membench``: the microbenchmark library instead), or ``build_library()`` /
+``build_rows_module()``.  Both
 files are kept in-tree so that a process which loads them shows them among its mapped files.
 """
 from __future__ import annotations
@@ -33,16 +34,10 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
-APPROX_LIBRARY = os.path.join(HERE, "libfsadam_approx.so")
-
-
-def build_library(verbose: bool = False, experiment_approx: bool = False) -> str:
-    """Always recompiles; returns the path of the shared library.  ``experiment_approx``: build the measurement
-    variant with approximate division and square root into ``libfsadam_approx.so`` instead (never loaded by the
-    package unless ``FSADAM_LIBRARY`` names it; its results are NOT bit-identical to the oracle)."""
-    target = APPROX_LIBRARY if experiment_approx else LIBRARY
-    extra = ["-DFSADAM_EXPERIMENT_APPROX_DIV_SQRT"] if experiment_approx else []
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra, "-I", INCLUDE, "-I", HERE, "-o", target + ".tmp", SOURCE]
+def build_library(verbose: bool = False) -> str:
+    """Always recompiles; returns the path of the shared library."""
+    target = LIBRARY
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", INCLUDE, "-I", HERE, "-o", target + ".tmp", SOURCE]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"  # the host pass does not know the device feature
     log = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
@@ -58,8 +53,14 @@ MEMBENCH_SOURCE = os.path.join(HERE, "membench.hip")
 MEMBENCH_LIBRARY = os.path.join(HERE, "libfsadam_membench.so")
 
 
+def membench_is_current() -> bool:
+    """The microbenchmark library is there and not older than its source."""
+    return os.path.exists(MEMBENCH_LIBRARY) and os.path.getmtime(MEMBENCH_LIBRARY) >= os.path.getmtime(MEMBENCH_SOURCE)
+
+
 def build_membench(verbose: bool = False) -> str:
-    """The microbenchmark kernels of ``bench.py --micro`` (a library of their own: nothing in the product loads it)."""
+    """The microbenchmark kernels of ``bench.py --micro`` and the copy kernel of ``bench.py --calib-copy-bytes`` (a library
+    of their own: nothing in the product loads it, and it is built when one of those two asks for it)."""
     cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", MEMBENCH_LIBRARY + ".tmp", MEMBENCH_SOURCE]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     noise = "is not a recognized feature for this target"
@@ -110,9 +111,8 @@ def build_rows_module(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    if "--experiment-approx" in sys.argv[1:]:
-        print(build_library(verbose=True, experiment_approx=True))
+    if "--membench" in sys.argv[1:]:  # the microbenchmark kernels only (bench.py --micro builds them itself when they are missing)
+        print(build_membench(verbose=True))
         sys.exit(0)
     print(build_library(verbose=True))
-    print(build_membench(verbose=True))
     print(build_rows_module(verbose=True))

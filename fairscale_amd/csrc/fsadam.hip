@@ -1345,17 +1345,4 @@ int fsadam_clear_cache(void) {
     return FSADAM_OK;
 }
 
-int fsadam_calib_copy(void* dst, const void* src, int64_t nbytes, void* hip_stream) {
-    if (!dst || !src || nbytes < 0 || (nbytes & 15) || !aligned_to(dst, 16) || !aligned_to(src, 16))
-        return fail(FSADAM_EINVAL, "calib copy needs 16-byte aligned pointers and a multiple of 16 bytes");
-    if (nbytes == 0) return FSADAM_OK;
-    const int64_t quads = nbytes / 16;
-    const int64_t grid = ceil_div(quads, 64);
-    if (grid > 0x7fffffff) return fail(FSADAM_EINVAL, "calib copy larger than 2^31 wavefronts");
-    hipLaunchKernelGGL(fsadam_copy_kernel<64>, dim3((uint32_t)grid), dim3(64), 20480, static_cast<hipStream_t>(hip_stream),
-                       static_cast<f32x4*>(dst), static_cast<const f32x4*>(src), quads);
-    FS_HIP(hipGetLastError());
-    return FSADAM_OK;
-}
-
 }  // extern "C"

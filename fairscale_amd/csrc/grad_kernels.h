@@ -1,5 +1,4 @@
-// Device code of the pre-step gradient pass (fsadam_grad_tiles, its two reduction kernels) and the
-// plain copy kernel used to calibrate the profiler's traffic counters.
+// Device code of the pre-step gradient pass (fsadam_grad_tiles, its two reduction kernels).
 // Included by fsadam.hip only (one translation unit).
 #pragma once
 
@@ -306,16 +305,6 @@ __global__ __launch_bounds__(64) void fsadam_put_descs(ChunkDesc* __restrict__ t
     gptr<uint32_t> out = (gptr<uint32_t>)reinterpret_cast<uint32_t*>(table + first);
     const uint32_t* in = reinterpret_cast<const uint32_t*>(batch.rows);
     for (uint32_t w = threadIdx.x; w < count * kWords; w += 64) out[w] = in[w];
-}
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-template <int BLOCK>
-__global__ __launch_bounds__(BLOCK) void fsadam_copy_kernel(f32x4* __restrict__ dst_, const f32x4* __restrict__ src_, int64_t n_quads) {
-    gptr<f32x4> dst = (gptr<f32x4>)dst_;
-    gptr<const f32x4> src = (gptr<const f32x4>)src_;
-    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    if (i < n_quads) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 }  // namespace

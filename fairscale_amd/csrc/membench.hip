@@ -129,6 +129,12 @@ __global__ __launch_bounds__(64) void mb_table_lds(const MbDesc* table, uint32_t
     st<true>(p, a);
 }
 
+// ---- variants 30-33: the two ways to the descriptor again, with the stores written through (sc1 nt) as the Adam kernels
+// issue them, for the 28-byte shape (30 scalar load, 31 staged in LDS) and the MEMORY_EFFICIENT shape (32, 33; the table
+// then holds p and g advanced as fp16 streams, see mb_fill_table).  Defined after st_policy below.
+template <bool LDS, bool MEMEFF>
+__global__ __launch_bounds__(64) void mb_table_through(const MbDesc* table, uint32_t log2_tiles);
+
 // ---- variants 5/6: the fp32 streams one direction at a time (one-shot tiles).
 __global__ __launch_bounds__(64) void mb_read4(const f4* p_, const f4* m_, const f4* v_, const f4* g_, int64_t nq, float* sink) {
     const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
@@ -353,7 +359,7 @@ __global__ __launch_bounds__(64) void mb_memeff_both_phased(f2* p_, f4* m_, f4* 
 #define MB_POLICY_CASES(X) X(0, "") X(1, " sc0") X(2, " sc1") X(3, " sc0 sc1") X(4, " nt") X(5, " sc0 nt") X(6, " sc1 nt") X(7, " sc0 sc1 nt")
 template <int POLICY>
 __device__ __forceinline__ void st_policy(FS_GLOBAL f4* p, f4 v) {
-#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_store_dwordx4 %0, %1, off" BITS ::"v"(p), "v"(v) : "memory");
+#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_store_dwordx4 %0, %1, off" BITS "\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
     MB_POLICY_CASES(X)
 #undef X
 }
@@ -363,15 +369,19 @@ __device__ __forceinline__ void st_policy(FS_GLOBAL f2* p, f2 v) {
     MB_POLICY_CASES(X)
 #undef X
 }
+// The four loads of a MEMORY_EFFICIENT tile and the wait for them in ONE statement: the compiler neither counts loads it
+// did not issue nor knows when their results arrive, so nothing may sit between them and their wait (outputs are
+// early-clobber: no result register doubles as an address).
 template <int POLICY>
-__device__ __forceinline__ void ld_policy(f4& out, FS_GLOBAL const f4* p) {
-#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_load_dwordx4 %0, %1, off" BITS : "=v"(out) : "v"(p) : "memory");
-    MB_POLICY_CASES(X)
-#undef X
-}
-template <int POLICY>
-__device__ __forceinline__ void ld_policy(f2& out, FS_GLOBAL const f2* p) {
-#define X(N, BITS) if constexpr (POLICY == N) asm volatile("global_load_dwordx2 %0, %1, off" BITS : "=v"(out) : "v"(p) : "memory");
+__device__ __forceinline__ void ld4_policy(f2& a, f2& d, f4& b, f4& c, FS_GLOBAL const f2* pa, FS_GLOBAL const f2* pd, FS_GLOBAL const f4* pb,
+                                           FS_GLOBAL const f4* pc) {
+#define X(N, BITS)                                                                                                                        \
+    if constexpr (POLICY == N)                                                                                                            \
+        asm volatile("global_load_dwordx2 %0, %4, off" BITS "\n\tglobal_load_dwordx2 %1, %5, off" BITS "\n\tglobal_load_dwordx4 %2, %6, off" BITS \
+                     "\n\tglobal_load_dwordx4 %3, %7, off" BITS "\n\ts_waitcnt vmcnt(0)"                                               \
+                     : "=&v"(a), "=&v"(d), "=&v"(b), "=&v"(c)                                                                              \
+                     : "v"(pa), "v"(pd), "v"(pb), "v"(pc)                                                                                  \
+                     : "memory");
     MB_POLICY_CASES(X)
 #undef X
 }
@@ -387,13 +397,7 @@ __global__ __launch_bounds__(64) void mb_memeff_both_policy(f2* p_, f4* m_, f4* 
         b = ld<true>((FS_GLOBAL const f4*)m_ + i);
         c = ld<true>((FS_GLOBAL const f4*)v_ + i);
     } else {
-        ld_policy<LOADS>(a, (FS_GLOBAL const f2*)p_ + i);
-        ld_policy<LOADS>(d, (FS_GLOBAL const f2*)g_ + i);
-        ld_policy<LOADS>(b, (FS_GLOBAL const f4*)m_ + i);
-        ld_policy<LOADS>(c, (FS_GLOBAL const f4*)v_ + i);
-        // the compiler does not count loads it did not issue: wait for them here, with the values as operands so that
-        // nothing that uses them moves in front
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(d), "+v"(b), "+v"(c)::"memory");
+        ld4_policy<LOADS>(a, d, b, c, (FS_GLOBAL const f2*)p_ + i, (FS_GLOBAL const f2*)g_ + i, (FS_GLOBAL const f4*)m_ + i, (FS_GLOBAL const f4*)v_ + i);
     }
     const f4 g = {d[0], d[1], d[0], d[1]};
     b = b * 0.9f + g * 0.1f;
@@ -408,6 +412,48 @@ __global__ __launch_bounds__(64) void mb_memeff_both_policy(f2* p_, f4* m_, f4* 
         st_policy<STORES>((FS_GLOBAL f4*)m_ + i, b);
         st_policy<STORES>((FS_GLOBAL f4*)v_ + i, c);
         st_policy<STORES>((FS_GLOBAL f2*)p_ + i, a);
+    }
+}
+
+template <bool LDS, bool MEMEFF>
+__global__ __launch_bounds__(64) void mb_table_through(const MbDesc* table, uint32_t log2_tiles) {
+    const uint32_t chunk = blockIdx.x >> log2_tiles, tile = blockIdx.x & ((1u << log2_tiles) - 1u);
+    MbDesc d;
+    if constexpr (LDS) {
+        __shared__ MbDesc staged;
+        if (threadIdx.x < 16) reinterpret_cast<uint32_t*>(&staged)[threadIdx.x] = reinterpret_cast<const uint32_t*>(table + chunk)[threadIdx.x];
+        __syncthreads();
+        d = staged;
+    } else {
+        typedef uint32_t words_t __attribute__((ext_vector_type(16)));
+        const words_t raw = *reinterpret_cast<const __attribute__((address_space(4))) words_t*>((const __attribute__((address_space(4))) MbDesc*)table + chunk);
+        d = __builtin_bit_cast(MbDesc, raw);
+    }
+    const uint64_t i = (uint64_t)tile * 64 + threadIdx.x;
+    if (i >= d.nq) return;
+    FS_GLOBAL f4* m = (FS_GLOBAL f4*)d.m + i;
+    FS_GLOBAL f4* v = (FS_GLOBAL f4*)d.v + i;
+    if constexpr (MEMEFF) {
+        FS_GLOBAL f2* p = (FS_GLOBAL f2*)reinterpret_cast<f2*>(d.p) + i;
+        f2 a = ld<true>((FS_GLOBAL const f2*)p);
+        const f2 e = ld<true>((FS_GLOBAL const f2*)reinterpret_cast<const f2*>(d.g) + i);
+        f4 b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v);
+        const f4 g = {e[0], e[1], e[0], e[1]};
+        b = b * 0.9f + g * 0.1f;
+        c = c * 0.999f + g * g * 0.001f;
+        a[0] -= b[0] * 0.001f;
+        a[1] -= b[1] * 0.001f;
+        st_policy<6>(m, b);
+        st_policy<6>(v, c);
+        st_policy<6>(p, a);
+    } else {
+        FS_GLOBAL f4* p = (FS_GLOBAL f4*)d.p + i;
+        f4 a = ld<true>((FS_GLOBAL const f4*)p), b = ld<true>((FS_GLOBAL const f4*)m), c = ld<true>((FS_GLOBAL const f4*)v),
+           e = ld<true>((FS_GLOBAL const f4*)d.g + i);
+        fake_update(a, b, c, e);
+        st_policy<6>(m, b);
+        st_policy<6>(v, c);
+        st_policy<6>(p, a);
     }
 }
 
@@ -519,13 +565,21 @@ __global__ __launch_bounds__(64) void mb_memeff_half_tile(float* p_, f2* m_, f2*
     asm volatile("global_store_dword %0, %1, off sc1 nt" ::"v"((FS_GLOBAL float*)p_ + i), "v"(a) : "memory");
 }
 
+__global__ __launch_bounds__(64) void mb_copy(f4* dst_, const f4* src_, int64_t n_quads) {
+    const int64_t i = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (i < n_quads) __builtin_nontemporal_store(__builtin_nontemporal_load((FS_GLOBAL const f4*)src_ + i), (FS_GLOBAL f4*)dst_ + i);
+}
+
 // fills a table of descriptors over four flat buffers, `chunk_q` quads each (runs once, outside the timing)
-__global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc) {
+// half_pg: p and g are fp16 streams (8 bytes per group of four elements), as in the MEMORY_EFFICIENT shape
+__global__ void mb_fill_table(MbDesc* table, f4* p, f4* m, f4* v, const f4* g, uint64_t nq, uint64_t chunk_q, uint32_t n_desc, int half_pg) {
     const uint32_t k = blockIdx.x * blockDim.x + threadIdx.x;
     if (k >= n_desc) return;
     const uint64_t first = (uint64_t)k * chunk_q;
     MbDesc d = {};
-    d.p = p + first; d.m = m + first; d.v = v + first; d.g = g + first;
+    d.m = m + first; d.v = v + first;
+    if (half_pg) { d.p = reinterpret_cast<f4*>(reinterpret_cast<f2*>(p) + first); d.g = reinterpret_cast<const f4*>(reinterpret_cast<const f2*>(g) + first); }
+    else { d.p = p + first; d.g = g + first; }
     d.nq = nq - first < chunk_q ? nq - first : chunk_q;
     table[k] = d;
 }
@@ -550,7 +604,8 @@ int64_t fsadam_membench_table_bytes(int64_t numel) {
 // Launches variant `kind` once over `numel` elements (a multiple of 4) on `stream`.  p, m, v, g: device buffers of
 // numel floats (the MEMORY_EFFICIENT variants use the first half of p and g as fp16).  lds_bytes: untouched LDS given to
 // every workgroup (caps residency).  param: variant 1: workgroups per compute unit; variants 14-16: log2 of the run length in tiles; variants 17-19: the period in 10 ns ticks.  table: device memory of
-// fsadam_membench_table_bytes(numel) bytes for variants 3, 4 and -1 (-1 fills it; do that once before them).
+// fsadam_membench_table_bytes(numel) bytes for variants 3, 4, 30-33, -1 and -2 (-1 fills it for the fp32 shape, -2 for the
+// MEMORY_EFFICIENT shape of variants 32 and 33; do that before them).
 // Returns 0, or -1 for an unknown kind / bad argument, -2 for a launch error.
 int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t numel, int lds_bytes, int param, void* table, void* sink,
                            void* stream_) {
@@ -566,9 +621,23 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
     const uint32_t n_desc = (uint32_t)((nq + chunk_q - 1) / chunk_q);
     switch (kind) {
         case -1:
+        case -2:
             if (!table) return -1;
-            hipLaunchKernelGGL(mb_fill_table, dim3((n_desc + 255) / 256), dim3(256), 0, stream, (MbDesc*)table, P, M, V, G, (uint64_t)nq, (uint64_t)chunk_q, n_desc);
+            hipLaunchKernelGGL(mb_fill_table, dim3((n_desc + 255) / 256), dim3(256), 0, stream, (MbDesc*)table, P, M, V, G, (uint64_t)nq, (uint64_t)chunk_q, n_desc,
+                               kind == -2 ? 1 : 0);
             break;
+        case 30:
+        case 31:
+        case 32:
+        case 33: {
+            if (!table) return -1;
+            const uint32_t log2_tiles = 10, grid = n_desc << log2_tiles;
+            if (kind == 30) hipLaunchKernelGGL((mb_table_through<false, false>), dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            else if (kind == 31) hipLaunchKernelGGL((mb_table_through<true, false>), dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            else if (kind == 32) hipLaunchKernelGGL((mb_table_through<false, true>), dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            else hipLaunchKernelGGL((mb_table_through<true, true>), dim3(grid), dim3(64), lds, stream, (const MbDesc*)table, log2_tiles);
+            break;
+        }
         case 0: hipLaunchKernelGGL(mb_oneshot<true>, dim3((uint32_t)grid64), dim3(64), lds, stream, P, M, V, G, nq); break;
         case 1: {
             int dev = 0, cus = 256;
@@ -675,6 +744,18 @@ int fsadam_membench_launch(int kind, void* p, void* m, void* v, void* g, int64_t
         }
         default: return -1;
     }
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+// A plain 128-bit copy of known traffic (nbytes read + nbytes written), one wave64 per workgroup: what the profiler's
+// FETCH_SIZE / WRITE_SIZE counters are scaled by (bench.py --calib-copy-bytes).  nbytes must be a multiple of 16 and both
+// pointers 16-byte aligned.  Returns 0, -1 for a bad argument, -2 for a launch error.
+int fsadam_membench_copy(void* dst, const void* src, int64_t nbytes, void* stream_) {
+    if (!dst || !src || nbytes < 0 || (nbytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15)) return -1;
+    if (nbytes == 0) return 0;
+    const int64_t quads = nbytes / 16, grid = (quads + 63) / 64;
+    if (grid > 0x7fffffff) return -1;
+    hipLaunchKernelGGL(mb_copy, dim3((uint32_t)grid), dim3(64), 20480, static_cast<hipStream_t>(stream_), (f4*)dst, (const f4*)src, quads);
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 

@@ -23,8 +23,8 @@ Deliberate differences, all supersets of the reference behaviour:
   copy, adam.py:128, and never reads it).
 * ``exp_avg``/``exp_avg_sq`` are laid out like the parameters (``zeros_like`` per parameter in the reference,
   adam.py:226-228): parameters that are back-to-back views of one buffer (OSS's buckets, oss.py:630-659) get
-  state that is back-to-back views of one buffer too, and so do the fp32 master copies of MIXED_PRECISION; a
-  run that starts between 128-byte lines gets state that starts as many elements past a line.  The native
+  state that is back-to-back views of one buffer too, and so do the fp32 master copies of MIXED_PRECISION; the
+  state of a run of 8192 elements or more starts as many elements past a 1 KiB boundary as the run does.  The native
   layout then treats each run as one tensor.  The placement is re-established (one copy of the state) after
   ``load_state_dict`` and after ``optimizer.state[p]`` has been assigned directly, as
   ``OSS.load_state_dict`` does (oss.py:453-461).
@@ -33,7 +33,6 @@ from __future__ import annotations
 
 from collections import defaultdict
 from enum import Enum, auto
-from operator import is_not
 from typing import Any, Callable, Dict, List, Optional, Tuple, Union
 
 import torch
@@ -88,29 +87,41 @@ def _adjacent_runs(tensors: List[torch.Tensor]) -> List[List[int]]:
     return runs
 
 
-def _needs_offset(first: torch.Tensor, total: int) -> bool:
-    """A run of ``total`` elements starting at ``first`` whose tiles the native layout moves onto line boundaries
-    by splitting off a head: its other streams must then leave their lines at the same element."""
-    return total >= _PLACE_MIN and first.data_ptr() % 128 != 0
+def _phase(t: torch.Tensor) -> int:
+    """Where a tensor starts, in elements past a boundary of 512 elements (1 KiB of fp16, 2 KiB of fp32)."""
+    return (t.data_ptr() // t.element_size()) % 512
+
+
+def _needs_placing(total: int) -> bool:
+    """A run of ``total`` elements is long enough for the native layout to split off a head, so that the tiles behind it
+    start on 1 KiB boundaries: the streams that accompany the run must then share its phase.  A wave moves 512 or 1024
+    contiguous bytes of a stream per instruction, and a stream that is on a 128-byte line but off a 1 KiB boundary costs
+    1.5 % of the step's rate (all four: 5 %); the allocator hands out 512-byte granules, so without this every stream of a
+    separately allocated tensor has even odds of being off."""
+    return total >= _PLACE_MIN
 
 
 def _buffer_placed_like(first: torch.Tensor, total: int, dtype: torch.dtype, zero: bool) -> torch.Tensor:
-    """``total`` elements of ``dtype`` for a stream that accompanies a run starting at ``first``.  A run that
-    starts between cache lines gets a stream that starts as many elements past a 1 KiB boundary as it does,
-    modulo 512, inside an allocation 512 elements longer: the native layout then finds ONE head length that
-    puts the tiles of both on line boundaries."""
+    """``total`` elements of ``dtype`` for a stream that accompanies a run starting at ``first``.  For a run long enough to
+    be given a head, the stream starts as many elements past a boundary of 512 elements as the run does (which may be
+    none): the native layout then finds ONE head length that puts the tiles of both on 1 KiB boundaries, wherever the
+    allocator put the run.  Taken from a plain allocation when that happens to have the right phase, else from one 512
+    elements longer."""
     make = torch.zeros if zero else torch.empty
-    if not _needs_offset(first, total):
+    if not _needs_placing(total):
         return make(total, dtype=dtype, device=first.device)
-    want = (first.data_ptr() // first.element_size()) % 512
+    want = _phase(first)
+    buf = torch.empty(total, dtype=dtype, device=first.device)
+    if _phase(buf) == want:
+        return buf.zero_() if zero else buf
+    del buf
     buf = make(total + 512, dtype=dtype, device=first.device)
-    have = (buf.data_ptr() // buf.element_size()) % 512
-    start = (want - have) % 512
+    start = (want - _phase(buf)) % 512
     return buf[start:start + total]
 
 
 def _placed(streams: List[torch.Tensor], likes: List[torch.Tensor]) -> bool:
-    """Do ``streams`` (one per entry of the run ``likes``) already lie back to back, at the run's offset?"""
+    """Do ``streams`` (one per entry of the run ``likes``) already lie back to back, at the run's phase?"""
     first, total = likes[0], sum(t.numel() for t in likes)
     end = None
     for st, like in zip(streams, likes):
@@ -121,8 +132,8 @@ def _placed(streams: List[torch.Tensor], likes: List[torch.Tensor]) -> bool:
         if end is not None and st.data_ptr() != end:
             return False
         end = st.data_ptr() + st.numel() * st.element_size()
-    if _needs_offset(first, total):
-        return (streams[0].data_ptr() // streams[0].element_size()) % 512 == (first.data_ptr() // first.element_size()) % 512
+    if _needs_placing(total):
+        return _phase(streams[0]) == _phase(first)
     return True
 
 
@@ -180,6 +191,11 @@ class Adam(torch.optim.Optimizer):
 
     state: dict
     defaults: dict
+    # Lay ``exp_avg`` / ``exp_avg_sq`` (and the fp32 master copies) out like the parameters: see ``_place_state``.  With
+    # False (set it on the class before constructing an optimizer, or on an instance before its first step) every
+    # parameter gets state from an allocation of its own, as ``zeros_like`` gives it in the reference (adam.py:226-228):
+    # for code that pickles, frees or replaces the state of single parameters and counts on each tensor owning its storage.
+    place_state: bool = True
 
     def __init__(
         self,
@@ -248,9 +264,9 @@ class Adam(torch.optim.Optimizer):
         params = list(params)
         masters: List[Any] = [None] * len(params)
         datas = [p.data for p in params]
-        for run in _adjacent_runs(datas):
+        for run in (_adjacent_runs(datas) if self.place_state else [[k] for k in range(len(datas))]):
             likes = [datas[k] for k in run]
-            flat = _buffer_placed_like(likes[0], sum(t.numel() for t in likes), torch.float32, zero=False)
+            flat = self._stream_for(likes[0], sum(t.numel() for t in likes), torch.float32, zero=False)
             at = 0
             for k, like in zip(run, likes):
                 view = flat[at:at + like.numel()].view(like.shape)
@@ -261,6 +277,11 @@ class Adam(torch.optim.Optimizer):
         for name, default in self.defaults.items():
             group.setdefault(name, default)
         self.fp32_param_groups = [group]
+
+    def _stream_for(self, first: torch.Tensor, total: int, dtype: torch.dtype, zero: bool) -> torch.Tensor:
+        if not self.place_state:
+            return (torch.zeros if zero else torch.empty)(total, dtype=dtype, device=first.device)
+        return _buffer_placed_like(first, total, dtype, zero)
 
     @property
     def supports_memory_efficient_fp16(self) -> bool:
@@ -413,13 +434,13 @@ class Adam(torch.optim.Optimizer):
     def _place_state(self, states: List[dict], likes: List[torch.Tensor], fresh_copy: bool = False) -> None:
         """Give every state dict its ``exp_avg``/``exp_avg_sq``, laid out like the parameters: each run of
         parameters that lie back to back in memory gets state that lies back to back, starting as many
-        elements past a cache line as the run does.  Missing tensors are created as zeros (adam.py:226-228);
+        elements past a 1 KiB boundary as the run does.  Missing tensors are created as zeros (adam.py:226-228);
         tensors that are there but lie elsewhere (restored from a checkpoint, or assigned to
         ``optimizer.state[p]`` directly) are copied into place once.  State of another dtype, shape or device
         is left alone: the checks of the step name it.  ``fresh_copy``: the tensors in ``states`` belong to
         somebody else (a checkpoint): copy them even where they already lie right."""
         optim_type = self.optim_type
-        runs = _adjacent_runs(likes)
+        runs = _adjacent_runs(likes) if self.place_state else [[k] for k in range(len(likes))]
         # All first moments are allocated before the first second moment, so that exp_avg and exp_avg_sq of one
         # parameter do not end up exactly one tensor apart: a model's matrices tend to be powers of two in size
         # (4096 x 4096 halves = 32 MiB), and two streams of one tile a power of two apart fall onto the same DRAM
@@ -434,13 +455,13 @@ class Adam(torch.optim.Optimizer):
                        for t, like in zip(have, run_likes) if t is not None):
                     for k, like in zip(run, run_likes):  # foreign state: only fill the gaps
                         if states[k].get(key) is None:
-                            states[k][key] = _buffer_placed_like(like, like.numel(), optim_type, zero=True).view(like.shape)
+                            states[k][key] = self._stream_for(like, like.numel(), optim_type, zero=True).view(like.shape)
                         elif fresh_copy:
                             states[k][key] = states[k][key].clone()
                     continue
-                if len(there) == len(have) and not fresh_copy and _placed(have, run_likes):
+                if len(there) == len(have) and not fresh_copy and (not self.place_state or _placed(have, run_likes)):
                     continue
-                flat = _buffer_placed_like(run_likes[0], total, optim_type, zero=len(there) < len(have))
+                flat = self._stream_for(run_likes[0], total, optim_type, zero=len(there) < len(have))
                 at = 0
                 for k, like, old in zip(run, run_likes, have):
                     view = flat[at:at + like.numel()].view(like.shape)
@@ -467,7 +488,7 @@ class Adam(torch.optim.Optimizer):
     def _gather_native(self, gi: int, group: Dict[str, Any], native_mode: int):
         """The steady-state walk in one C++ loop (csrc/tensor_rows.cpp): gradients, state tensors,
         checks, pointers and step counters.  Returns (plan, table_changed, step) or None when the
-        helper is not built or anything is out of the ordinary; the Python walks then decide."""
+        helper is not built or anything is out of the ordinary; the general walk (``_gather``) then decides."""
         native = _rows.native
         if native is None:
             return None
@@ -493,45 +514,6 @@ class Adam(torch.optim.Optimizer):
             plan = self._plans[(gi, device)] = TensorListPlan(native_mode, device)
         return plan
 
-    def _gather_fast(self, gi: int, group: Dict[str, Any]):
-        """Same result as ``_gather`` for the steady state (every parameter of the group has a dense
-        gradient and an initialised state, all on one device) without the per-parameter dictionary
-        walk; returns (None, None) when that does not hold and the general walk must run."""
-        cache = self._steady_group(gi, group)
-        if cache is None:
-            return None, None
-        params, snapshot, states, masters, outs, device, _, _, _ = cache
-        if any(map(is_not, params, snapshot)):
-            return None, None  # the list was edited in place: the collected states belong to other parameters
-        lists: List[List[torch.Tensor]] = [[] for _ in range(5 if (masters is not None or outs is not None) else 4)]
-        taking_part = []
-        for pj, (p, st) in enumerate(zip(params, states)):
-            g = p.grad
-            if st is None:
-                if g is not None:
-                    return None, None  # a parameter that sat out has a gradient now
-                continue
-            if g is None or g.is_sparse:
-                return None, None
-            try:
-                lists[1].append(st["exp_avg"])
-                lists[2].append(st["exp_avg_sq"])
-                st["step"]
-            except KeyError:  # a state dict was emptied behind our back: let the general walk re-initialise it
-                return None, None
-            lists[0].append(masters[pj] if masters is not None else p)
-            lists[3].append(g)
-            if masters is not None:
-                lists[4].append(p)
-            elif outs is not None:
-                lists[4].append(outs[pj])
-            taking_part.append(st)
-        if not taking_part:
-            return None, None
-        for st in taking_part:
-            st["step"] += 1
-        return {device: lists}, taking_part[-1]["step"]
-
     def _launch_group(self, gi: int, group: Dict[str, Any], native_mode: int, watch_overflow: bool, scale, flags: List[torch.Tensor]) -> None:
         """Walk one parameter group and enqueue its step (adam.py:202-276); the flags to read back are appended to ``flags``."""
         beta1, beta2 = group["betas"]
@@ -546,9 +528,7 @@ class Adam(torch.optim.Optimizer):
             plan.step_rows(table_changed, group["lr"], beta1, beta2, group["eps"], scale, self._optim_scale, flag,
                            step_no, self.eps_mode, bias_correction, group["weight_decay"])
             return
-        batches, step_no = self._gather_fast(gi, group)
-        if batches is None:
-            batches, step_no = self._gather(gi, group)
+        batches, step_no = self._gather(gi, group)
         if not batches:
             # adam.py:256 indexes the first device of an empty dict
             raise IndexError("list index out of range")

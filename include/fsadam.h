@@ -275,12 +275,6 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
 /* Drops the tables cached by fsadam_step and fsadam_grad_pass (synchronises the devices that own them). */
 int fsadam_clear_cache(void);
 
-/* ---- measurement aid: a plain 128-bit copy kernel of known traffic (nbytes read + nbytes
- * written), used to calibrate the profiler's FETCH_SIZE / WRITE_SIZE counters and as the
- * achievable-bandwidth yardstick next to the Adam kernels.  nbytes must be a multiple of 16 and
- * both pointers 16-byte aligned. */
-int fsadam_calib_copy(void* dst, const void* src, int64_t nbytes, void* hip_stream);
-
 #ifdef __cplusplus
 }
 #endif

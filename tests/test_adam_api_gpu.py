@@ -530,6 +530,47 @@ def test_parameters_packed_into_a_flat_buffer_step_like_separate_ones(api, cuda_
             assert torch.equal(fresh.state[q][key], opts[1].state[q][key])
 
 
+@pytest.mark.parametrize("precision_name", ["FULL_PRECISION", "MEMORY_EFFICIENT_MIXED_PRECISION", "PURE_FP16", "MIXED_PRECISION"])
+def test_state_of_separately_allocated_parameters_shares_their_phase_unless_switched_off(api, cuda_device, precision_name):
+    """The allocator hands out 512-byte granules, so a parameter of its own starts on a 1 KiB boundary or half a
+    kilobyte past one: its state (and fp32 master copy) starts the same number of elements past a boundary of 512
+    elements, so that ONE head puts every stream the optimizer owns on 1 KiB boundaries.  With ``place_state`` off every
+    state tensor owns an allocation of exactly its size, as ``zeros_like`` gives it in the reference
+    (adam.py:226-228), and a single parameter's state pickles to its own size.  Same values either way."""
+    Adam, _, Precision = api
+    sizes = (8192, 70001, 9000, 33, 20480, 131072 + 128)
+    keep = [torch.empty(128, device=cuda_device) for _ in range(3)]  # shift the allocator's phase between the lists
+    a = _random_problem(precision_name, cuda_device, sizes)
+    b = [p.detach().clone().requires_grad_() for p in a]
+    placed = Adam(a, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name])
+    plain = Adam(b, lr=1e-2, weight_decay=0.01, precision=Precision[precision_name])
+    plain.place_state = False
+    if precision_name == "MIXED_PRECISION":  # the master copies were made by the constructor: make them again, unplaced
+        plain._build_fp32_params(b)
+    for step in range(1, 4):
+        _set_grads(a, step)
+        for p, q in zip(a, b):
+            q.grad = p.grad.clone()
+        placed.step()
+        plain.step()
+    phase = lambda t: (t.data_ptr() // t.element_size()) % 512  # noqa: E731
+    for j, (p, q) in enumerate(zip(a, b)):
+        assert torch.equal(p.detach(), q.detach())
+        like = placed.fp32_param_groups[0]["params"][j] if precision_name == "MIXED_PRECISION" else p
+        if precision_name == "MIXED_PRECISION" and p.numel() >= 8192:
+            assert phase(like) == phase(p)
+        for key in ("exp_avg", "exp_avg_sq"):
+            assert torch.equal(placed.state[p][key], plain.state[q][key])
+            if p.numel() >= 8192:
+                assert phase(placed.state[p][key]) == phase(like), (j, key)
+            own = plain.state[q][key]
+            assert own.untyped_storage().nbytes() == own.numel() * own.element_size() and own.storage_offset() == 0
+        blob = io.BytesIO()
+        torch.save(plain.state[q], blob)
+        assert blob.getbuffer().nbytes < 2 * q.numel() * plain.state[q]["exp_avg"].element_size() + 4096
+    del keep
+
+
 # ---- runs: parameters that are back-to-back views of one buffer (oss.py:630-659, param_bucket.py:62-90)
 
 def _packed_problem(precision_name, device, sizes, lead=3, seed=5):

@@ -451,8 +451,6 @@ def test_plan_lifecycle_without_a_device():
     _cabi.check(L.fsadam_plan_destroy(handle))
     _cabi.check(L.fsadam_plan_destroy(None))
     _cabi.check(L.fsadam_clear_cache())
-    assert L.fsadam_calib_copy(None, None, 16, None) == EINVAL
-    assert L.fsadam_calib_copy(ctypes.c_void_p(4096), ctypes.c_void_p(8192), 24, None) == EINVAL
 
 
 # ---- the Python face of the native call (validation of multi_tensor_apply.cuh:49-67, dispatch of kernel.cu:165-263)
@@ -545,10 +543,25 @@ def test_wide_assembly_stores_carry_their_wait_states():
 
     src_dir = os.path.join(REPO, "fairscale_amd", "csrc")
     wide = 0
-    for path in glob.glob(os.path.join(src_dir, "fsadam*.h")) + glob.glob(os.path.join(src_dir, "*_kernels.h")) + [os.path.join(src_dir, "fsadam.hip")]:
+    sources = (glob.glob(os.path.join(src_dir, "fsadam*.h")) + glob.glob(os.path.join(src_dir, "*_kernels.h"))
+               + [os.path.join(src_dir, "fsadam.hip"), os.path.join(src_dir, "membench.hip")])  # the microbenchmarks too: their figures decide shapes
+    for path in sources:
         text = open(path).read()
         for statement in re.findall(r'asm volatile\((.*?)\);', text, flags=re.S):
             if "global_store_dwordx4" in statement or "global_store_dwordx3" in statement:
                 wide += 1
-                assert re.search(r'global_store_dwordx[34][^"]*\\n\\ts_nop 1"', statement), f"{path}: a wide store without its wait states"
-    assert wide >= 1
+                after = statement[re.search(r'global_store_dwordx[34]', statement).end():]
+                assert re.search(r'\\n\\ts_nop 1"', after), f"{path}: a wide store without its wait states"
+    assert wide >= 2
+
+
+def test_assembly_loads_wait_in_their_own_statement():
+    """A load issued from inline assembly is not counted by the compiler, which may therefore read (copy, spill) the
+    result register before the data has arrived unless the statement that issues the load also waits for it."""
+    import re
+
+    for name in ("membench.hip", "fsadam.hip", "fsadam_common.h", "adam_kernels.h", "grad_kernels.h"):
+        text = open(os.path.join(REPO, "fairscale_amd", "csrc", name)).read()
+        for statement in re.findall(r'asm volatile\((.*?)\);', text, flags=re.S):
+            if "global_load" in statement:
+                assert "s_waitcnt vmcnt(0)" in statement, f"{name}: a load from assembly without its wait"

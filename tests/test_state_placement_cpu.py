@@ -35,24 +35,37 @@ def test_adjacent_runs_follow_the_memory_not_the_list():
     assert A._adjacent_runs([flat[1:10], empty, flat[10:20]]) == [[0, 1, 2]]    # an empty view continues the run
 
 
-def test_a_stream_for_a_run_starts_where_the_run_leaves_its_cache_line():
+def test_a_stream_for_a_run_starts_at_the_runs_phase():
     flat = torch.zeros(200_000)  # float32: 512 elements = 2 KiB
     base = flat.data_ptr() // 4
-    for lead in (1, 3, 31, 100, 511, 513):
+    for lead in (0, 1, 3, 31, 100, 128, 256, 511, 513):  # 128 and 256 elements in: on a cache line, off the 1 KiB boundary
         first = flat[lead:lead + 50_000]
-        if first.data_ptr() % 128 == 0:
-            continue
         for dtype in (torch.float32, torch.float16):
             buf = A._buffer_placed_like(first, 50_000, dtype, zero=True)
             assert buf.numel() == 50_000 and buf.dtype == dtype and buf.is_contiguous() and not bool(buf.any())
-            # same element offset modulo 512: one head length aligns both
-            assert (buf.data_ptr() // buf.element_size()) % 512 == (base + lead) % 512
-    # short runs and runs that start on a line get a plain allocation
+            # same element offset modulo 512: one head length puts both on 1 KiB boundaries
+            assert A._phase(buf) == (base + lead) % 512 == A._phase(first)
+            buf = A._buffer_placed_like(first, 50_000, dtype, zero=False)
+            assert buf.numel() == 50_000 and A._phase(buf) == A._phase(first)
+    # short runs get a plain allocation, whatever their phase
     short = flat[1:1 + 100]
     assert A._buffer_placed_like(short, 100, torch.float32, zero=True).numel() == 100
-    on_line = (-(flat.data_ptr() // 4)) % 32  # host allocations are only 64-byte aligned: find a 128-byte boundary
-    assert not A._needs_offset(short, 100) and not A._needs_offset(flat[on_line:on_line + 50_000], 50_000)
-    assert A._needs_offset(flat[on_line + 1:on_line + 50_001], 50_000)
+    assert not A._needs_placing(100) and not A._needs_placing(8191) and A._needs_placing(8192)
+
+
+def test_a_run_on_a_boundary_gets_state_on_a_boundary():
+    """The allocator hands out 512-byte granules: state for a run that starts ON a 1 KiB boundary must not be left half a
+    kilobyte off it."""
+    flat = torch.zeros(100_000 + 1024)
+    lead = (-(flat.data_ptr() // 4)) % 512  # first element on a 2 KiB boundary
+    first = flat[lead:lead + 60_000]
+    assert A._phase(first) == 0
+    for _ in range(4):  # whatever the allocator returns
+        keep = torch.zeros(137)  # shift the allocator's next answer
+        for dtype in (torch.float32, torch.float16):
+            buf = A._buffer_placed_like(first, 60_000, dtype, zero=True)
+            assert A._phase(buf) == 0 and buf.data_ptr() % 1024 == 0
+        del keep
 
 
 def test_state_counts_as_placed_only_when_it_follows_the_parameters():
@@ -69,7 +82,7 @@ def test_state_counts_as_placed_only_when_it_follows_the_parameters():
     assert not A._placed([torch.zeros(n) for n in sizes], likes)                          # one allocation each
     assert not A._placed([good[0], good[1], torch.zeros(sizes[2])], likes)               # the last one elsewhere
     assert not A._placed([good[0], good[1], good[2][:-1]], likes)                         # a size that does not fit
-    # a short run, or one that starts on a line: packed is enough
+    # a short run: packed is enough
     small_likes = _views(params, [10, 20], lead=1)
     assert A._placed(_views(state, [10, 20], lead=7), small_likes)
 
