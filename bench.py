@@ -357,6 +357,14 @@ def measure_c5(torch, steps, warmup, device):
     wall, host, per_step = time_loop(torch, lambda i: opt.step(), steps, warmup)
     assert opt._optim_scale == 65536.0 and opt._steps_since_optim_scale_change == steps + warmup
     sp = spread(per_step)
+    # one step on its own behind 20 ms of an idle GPU, timed like the two single steps below (wall clock around the call
+    # and a synchronisation): what a step costs when the device has to come back from idling, with nothing else changed
+    torch.cuda.synchronize()
+    time.sleep(0.02)
+    t0 = time.perf_counter()
+    opt.step()
+    torch.cuda.synchronize()
+    after_idle_ms = (time.perf_counter() - t0) * 1e3
     # the overflow step
     cpu_gen = torch.Generator().manual_seed(5002)
     saved = []
@@ -392,7 +400,7 @@ def measure_c5(torch, steps, warmup, device):
            "overflow_step": {"ms": overflow_ms, "injected": "1 gradient element in 10^6 set to 6e4", "optim_scale_before": 65536.0,
                              "optim_scale_after": opt._optim_scale, "state_zeroed": zeroed,
                              "note": "step + blocking flag read-back + scale halved + m, v of all 291 tensors zeroed in place by one launch (27 GB written)"},
-           "clean_step_after_backoff_ms": after_ms,
+           "clean_step_after_backoff_ms": after_ms, "single_step_after_20ms_idle_ms": after_idle_ms,
            "note": "every step includes the blocking read-back of the overflow flag, as in the reference (adam.py:278)"}
     del opt, params, saved
     torch.cuda.empty_cache()
@@ -677,6 +685,7 @@ def main():
             if "overflow_step" in r:
                 configs[key]["overflow_step_ms"] = r["overflow_step"]["ms"]
                 configs[key]["clean_step_after_backoff_ms"] = r["clean_step_after_backoff_ms"]
+                configs[key]["single_step_after_20ms_idle_ms"] = r["single_step_after_20ms_idle_ms"]
     # the committed counter summary speaks for default options only
     traffic = load_traffic(workload) if not args.opt else None
     traffic_source = (f"profiles/{TRAFFIC_SUMMARIES[workload]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this workload at default options; "

@@ -100,17 +100,19 @@ struct Options {
 };
 
 // Residency that measured fastest with one wave64 per workgroup, one vector per lane per stream and stores that
-// are written through (store_through): about 36 KiB of loads in flight per compute unit, i.e. 9 waves of the
+// are written through (store_through): about 36-40 KiB of loads in flight per compute unit, i.e. 10 waves of the
 // 4 KiB-per-wave modes and 12 of the 3 KiB-per-wave ones.  The hardware hands out LDS in granules of 1280 bytes
 // (a sweep in steps of 256 bytes changes the rate only at multiples of 1280), so a ballast of B bytes allows
-// floor(128 / ceil(B / 1280)) workgroups per compute unit: 12 288 -> 12, 14 080 -> 11, 15 360 -> 10, 16 640 and
-// 17 920 -> 9, 19 200 -> 8; 13 and 15 cannot be had.  One wave more or less costs 0.3-1.5 points, two cost 2-4.
-int64_t default_lds_throttle(int mode) {
+// floor(128 / ceil(B / 1280)) workgroups per compute unit: 11 520 -> 14, 12 288 -> 12, 14 080 -> 11, 15 360 -> 10,
+// 16 640 and 17 920 -> 9, 19 200 -> 8; 13 and 15 cannot be had.  One wave more or less costs 0.3-1.5 points, two
+// cost 2-4.  The optimum hardly moves with the size of the list (swept from 1e7 to 6.7e9 elements in every mode):
+// only the smallest lists like one step more residency, which is worth 1-2 points there.
+int64_t default_lds_throttle(int mode, int64_t total_elems) {
     switch (mode) {
-        case FSADAM_FULL_PRECISION: return 16640;
-        case FSADAM_FULL_PRECISION_FP16_COPY: return 16640;
-        case FSADAM_MIXED_PRECISION: return 16640;
-        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return 12288;
+        case FSADAM_FULL_PRECISION:
+        case FSADAM_FULL_PRECISION_FP16_COPY: return total_elems < 20000000 ? 14080 : 15360;
+        case FSADAM_MIXED_PRECISION: return 15360;
+        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return total_elems < 50000000 ? 11520 : 12288;
         default: return 12288;
     }
 }
@@ -380,7 +382,8 @@ struct FsAdamPlan {
     int mode = 0;
     int device = -1;
     hipStream_t upload_stream = nullptr;  // the library's own, for tables (see upload_table)
-    Options opt;
+    Options opt;                     // as asked for when the table was set (lds_throttle may be -1: by mode and size)
+    int64_t lds_bytes = 0;           // the ballast the current table is stepped with
     Layout layout;
     std::vector<FsAdamTensor> rows;  // what the current table was built from
     std::vector<FsAdamTensor> runs;  // scratch of plan_set_tensors: the rows after merging
@@ -518,38 +521,39 @@ int64_t fill_descs(ChunkDesc* out, const FsAdamTensor& r, int mode, int64_t star
 }
 
 template <int MODE>
-int launch_tiles(const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf, hipStream_t stream) {
+int launch_tiles(const ChunkDesc* table, const Layout& L, int64_t lds_bytes, const StepScalars& s, float* found_inf, hipStream_t stream) {
     const int64_t n_blocks = L.blocks();
     if (n_blocks == 0) return FSADAM_OK;
     if (n_blocks > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
-    hipLaunchKernelGGL((fsadam_tiles<MODE, kBlock, 1>), dim3((uint32_t)n_blocks), dim3(kBlock), (size_t)opt.lds_throttle, stream, table, tile_map(L), s,
+    hipLaunchKernelGGL((fsadam_tiles<MODE, kBlock, 1>), dim3((uint32_t)n_blocks), dim3(kBlock), (size_t)lds_bytes, stream, table, tile_map(L), s,
                        found_inf);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
 
-int launch_mode(int mode, const ChunkDesc* table, const Layout& L, const Options& opt, const StepScalars& s, float* found_inf,
+int launch_mode(int mode, const ChunkDesc* table, const Layout& L, int64_t lds_bytes, const StepScalars& s, float* found_inf,
                 hipStream_t stream) {
 #define FS_MODE(M) \
-    case M: return launch_tiles<M>(table, L, opt, s, found_inf, stream)
+    case M: return launch_tiles<M>(table, L, lds_bytes, s, found_inf, stream)
     switch (mode) {
         FS_MODE(FSADAM_FULL_PRECISION);
         FS_MODE(FSADAM_MIXED_PRECISION);
         FS_MODE(FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION);
         FS_MODE(FSADAM_FULL_PRECISION_FP16_COPY);
-        default: return launch_tiles<FSADAM_PURE_FP16>(table, L, opt, s, found_inf, stream);
+        default: return launch_tiles<FSADAM_PURE_FP16>(table, L, lds_bytes, s, found_inf, stream);
     }
 #undef FS_MODE
 }
 
-// On failure the plan is left without tensors (plan_step refuses) rather than with a layout that does not
-// belong to the table on the device.
+// A list that does not pass validation changes nothing.  A failure later on (an allocation, a HIP call) leaves the
+// plan without tensors (plan_step refuses) rather than with a layout that does not belong to the table on the device.
 int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, hipStream_t stream) {
-    plan->rows.clear();
+    // a list that is refused outright leaves the plan with the table it had
     int rc = validate_rows(tensors, n, plan->mode);
     if (rc) return rc;
     rc = refuse_capture(stream);
     if (rc) return rc;
+    plan->rows.clear();  // from here on a failure leaves the plan without tensors
     int dev = -1;
     FS_HIP(hipGetDevice(&dev));
     if (plan->device != dev) {
@@ -560,11 +564,11 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
         std::lock_guard<std::mutex> lock(g_mutex);
         plan->opt = g_opt;
     }
-    if (plan->opt.lds_throttle < 0) plan->opt.lds_throttle = default_lds_throttle(plan->mode);
     build_runs(tensors, n, plan->mode, plan->opt.merge_runs != 0, plan->runs, nullptr);
     compute_heads(plan->runs, plan->mode, plan->opt, plan->heads);
     Layout L = compute_layout(plan->runs, plan->heads, plan->mode, plan->opt);
     for (int64_t t = 0; t < n; ++t) L.n_empty += tensors[t].numel == 0 ? 1 : 0;
+    const int64_t lds_bytes = plan->opt.lds_throttle >= 0 ? plan->opt.lds_throttle : default_lds_throttle(plan->mode, L.total_elems);
     const int64_t n_descs = L.descs();
     if (L.blocks() > 0x7ffffff0) return fail(FSADAM_EINVAL, "tensor list too large for one launch");
 
@@ -614,6 +618,7 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     }
     // everything went through: the plan now describes the new table
     plan->layout = L;
+    plan->lds_bytes = lds_bytes;
     plan->rows.assign(tensors, tensors + n);
     plan->current = (plan->current + 1) % kTableSlots;
     plan->uploads += 1;
@@ -650,7 +655,7 @@ int plan_step(FsAdamPlan* plan, float lr, float beta1, float beta2, float eps, f
     TableSlot& slot = plan->slots[plan->current];
     int rc = mark_order_after(slot.mark, stream);
     if (rc) return rc;
-    rc = launch_mode(plan->mode, slot.d_table, L, plan->opt, s, found_inf, stream);
+    rc = launch_mode(plan->mode, slot.d_table, L, plan->lds_bytes, s, found_inf, stream);
     if (rc) return rc;
     return mark_use(slot.mark, stream, plan->lazy_events);
 }
@@ -1184,7 +1189,7 @@ int fsadam_plan_info(const FsAdamPlan* plan, FsAdamPlanInfo* out) {
     out->grid = L.blocks();
     out->block = kBlock;
     out->n_runs = L.n_runs;
-    out->lds_throttle = plan->opt.lds_throttle;
+    out->lds_throttle = plan->lds_bytes;
     out->uploads = plan->uploads;
     return FSADAM_OK;
 }
@@ -1209,7 +1214,6 @@ int fsadam_step(const FsAdamTensor* tensors, int64_t n_tensors, int precision_mo
         std::lock_guard<std::mutex> lock(g_mutex);
         now = g_opt;
     }
-    if (now.lds_throttle < 0) now.lds_throttle = default_lds_throttle(precision_mode);
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     FsAdamPlan* hit = nullptr;
     FsAdamPlan* victim = nullptr;

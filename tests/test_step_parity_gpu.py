@@ -777,6 +777,36 @@ def test_the_library_refuses_a_stream_that_is_being_captured(cuda_device):
     assert float(t[0][0]) != 0.5
 
 
+def test_a_list_that_fails_validation_leaves_the_plans_table(cuda_device):
+    """A plan that holds a table and is handed a list with a NULL pointer refuses the list and goes on stepping the
+    table it has: validation comes before anything of the plan is touched."""
+    import ctypes
+
+    from fairscale_amd import _cabi
+
+    L = _cabi.lib()
+    t = [torch.full((5000,), x, device=cuda_device) for x in (0.5, 0.0, 0.0, 0.01)]
+    rows = (_cabi.FsAdamTensor * 1)()
+    rows[0].p, rows[0].m, rows[0].v, rows[0].g = (x.data_ptr() for x in t)
+    rows[0].numel = 5000
+    plan = ctypes.c_void_p()
+    _cabi.check(L.fsadam_plan_create(_cabi.FULL_PRECISION, ctypes.byref(plan)))
+    stream = int(torch.cuda.current_stream(cuda_device).cuda_stream)
+    try:
+        _cabi.check(L.fsadam_plan_set_tensors(plan, rows, 1, stream))
+        bad = (_cabi.FsAdamTensor * 1)()
+        bad[0].p, bad[0].m, bad[0].v, bad[0].g, bad[0].numel = t[0].data_ptr(), None, t[2].data_ptr(), t[3].data_ptr(), 5000
+        assert L.fsadam_plan_set_tensors(plan, bad, 1, stream) == -1 and b"NULL" in L.fsadam_last_error()
+        info = _cabi.FsAdamPlanInfo()
+        _cabi.check(L.fsadam_plan_info(plan, ctypes.byref(info)))
+        assert info.n_tensors == 1 and info.uploads == 1
+        _cabi.check(L.fsadam_plan_step(plan, 1e-3, 0.9, 0.999, 1e-8, 1.0, 1.0, 0.0, 1, 1, 1, None, stream))
+        torch.cuda.synchronize(cuda_device)
+        assert float(t[0][0]) != 0.5 and float(t[1][0]) != 0.0
+    finally:
+        _cabi.check(L.fsadam_plan_destroy(plan))
+
+
 def _window_check(oracle, mode, before, after, grads, windows, kw, what):
     """Re-run the oracle on [lo, hi) windows of the pre-step device state and compare with the
     post-step device state."""
