@@ -52,6 +52,8 @@ def parse_args():
     ap.add_argument("--numel", type=int, default=SHARD_NUMEL, help="parameters in the flat shard")
     ap.add_argument("--mode", default="MEMORY_EFFICIENT_MIXED_PRECISION", choices=list(BYTES_PER_PARAM))
     ap.add_argument("--no-also", action="store_true", help="skip the secondary measurements (other dtype combinations, gradient pass, ragged list)")
+    ap.add_argument("--also-only", action="append", default=[], metavar="KEY",
+                    help="of the secondary measurements run only those whose key under \"also\" starts with KEY (may be repeated)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-numel", type=int, default=1 << 26, help="sample size of the CPU baseline")
     ap.add_argument("--calib-copy-bytes", type=int, default=0,
@@ -61,6 +63,9 @@ def parse_args():
     ap.add_argument("--micro-numel", type=int, default=SHARD_NUMEL)
     ap.add_argument("--micro-data", default="random", choices=["random", "zeros"],
                     help="what the microbenchmark's buffers hold and its write-only kernels store (the bandwidth of this part depends on it)")
+    ap.add_argument("--lds-sweep", default="", metavar="BYTES,BYTES,...",
+                    help="instead of the benchmark: the kernel's rate on --numel parameters in --mode for each of these LDS ballasts "
+                         "(library option lds_throttle), one line each")
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="library tuning option (lds_throttle, merge_runs, align_heads, mid_tiles, ...)")
     return ap.parse_args()
 
@@ -455,6 +460,46 @@ def load_traffic(workload_key):
     return int(found.group(1)) if found else None
 
 
+def run_lds_sweep(torch, args, device):
+    """The kernel's rate on ONE set of tensors (a flat shard of --numel parameters in --mode, state allocated once by the
+    optimizer) for each LDS ballast of --lds-sweep: between two values only the plan is made anew, so that where the
+    allocator put the tensors does not enter the comparison.  Three series of back-to-back launches per value (K launches
+    between two events, K sized to about 100 ms), the best of them printed.  LDS is handed out in granules of 1280 bytes:
+    a ballast of B bytes allows floor(128 / ceil(B / 1280)) waves per compute unit."""
+    from fairscale_amd import _cabi
+    from fairscale_amd.optim import Adam, Precision
+
+    p, scale = make_shard(torch, args.mode, args.numel, device)
+    opt = Adam([p], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, precision=getattr(Precision, args.mode))
+    opt.step(scale=scale)
+    bpp = BYTES_PER_PARAM[args.mode]
+    launches = max(10, min(2000, int(0.1 * 6.7e12 / (args.numel * bpp))))
+    group = opt.param_groups[0]
+    for lds in (int(x) for x in args.lds_sweep.split(",")):
+        _cabi.set_option("lds_throttle", lds)
+        opt._plans_invalidate()
+        for _ in range(3):
+            opt.step(scale=scale)  # the first one makes the plan and sends the table
+        plan_obj = next(iter(opt._plans.values()))
+        flag = opt._flags.get(device)
+        done = opt.state[p]["step"]
+        best = None
+        for _ in range(3):
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(launches):
+                plan_obj.step_rows(False, group["lr"], group["betas"][0], group["betas"][1], group["eps"], scale, opt._optim_scale, flag,
+                                   done + 1 + i, opt.eps_mode, 1, group["weight_decay"])
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / launches
+            best = ms if best is None else min(best, ms)
+        waves = 128 // -(-lds // 1280) if lds > 0 else 0
+        print(f"{args.mode} numel {args.numel:>11d} ballast {lds:6d} B ({waves:2d} waves per CU): {best:9.4f} ms per launch "
+              f"= {args.numel * bpp / best / 1e6 / HBM_PEAK_GBS * 100:5.2f} % of the HBM peak", flush=True)
+
+
 def load_membench():
     """The microbenchmark library (fairscale_amd/csrc/membench.hip), compiled first when it is missing or older than its
     source: nothing in the product loads it, so the ordinary build leaves it out."""
@@ -621,6 +666,9 @@ def main():
     if args.micro:
         run_micro(torch, args, device)
         return
+    if args.lds_sweep:
+        run_lds_sweep(torch, args, device)
+        return
     if args.calib_copy_bytes > 0:
         import ctypes
 
@@ -639,28 +687,30 @@ def main():
 
     main_res = measure_gpu(torch, args.mode, args.numel, args.steps, args.warmup, device)
     also = {}
-    if not args.no_also:
-        # the other three dtype combinations on the same number of parameters
-        for mode in ("MIXED_PRECISION", "FULL_PRECISION", "PURE_FP16", "MEMORY_EFFICIENT_MIXED_PRECISION"):
-            if mode == args.mode:
-                continue
-            r = measure_gpu(torch, mode, args.numel, args.steps, args.warmup, device)
-            also[mode] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "step_ms_median": r["step_ms_median"],
-                          "kernel_ms": r["kernel_ms"], "kernel_ms_min": r["kernel_ms_min"], "kernel_ms_median": r["kernel_ms_median"],
-                          "kernel_ms_max": r["kernel_ms_max"], "bytes_per_param": r["bytes_per_param"], "achieved_gbs": r["achieved_gbs"],
-                          "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS,
-                          "frac_of_hbm_peak_through_adam_step": args.numel * r["bytes_per_param"] / r["ms_per_step"] / 1e6 / HBM_PEAK_GBS}
-    if not args.no_also:
-        also["grad_pass_fp16"] = measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)
-        # steps of 0.5-1.5 ms: at least 100 of them, so that one slow step does not make the wall-clock figure
-        short_steps = max(args.steps, 100)
-        also["ragged_4096_FULL_PRECISION"] = measure_ragged(torch, short_steps, args.warmup, device)
-        also["ragged_4096_packed_views_FULL_PRECISION"] = measure_ragged(torch, short_steps, args.warmup, device, packed=True)
-        also["ragged_4096_moving_gradients_FULL_PRECISION"] = measure_ragged(torch, short_steps, args.warmup, device, moving=True)
-        also["c2_gpt2_small_148_tensors_MIXED_PRECISION"] = measure_c2(torch, short_steps, args.warmup, device)
-        also["c5_llama7b_291_tensors_PURE_FP16"] = measure_c5(torch, min(args.steps, 10), min(args.warmup, 3), device)
-        if not args.no_cpu:
-            also["c1_flat_2pow20_FULL_PRECISION_10_steps"] = measure_c1(torch, device)
+    wanted = lambda key: not args.no_also and (not args.also_only or any(key.startswith(k) for k in args.also_only))  # noqa: E731
+    # the other three dtype combinations on the same number of parameters
+    for mode in ("MIXED_PRECISION", "FULL_PRECISION", "PURE_FP16", "MEMORY_EFFICIENT_MIXED_PRECISION"):
+        if mode == args.mode or not wanted(mode):
+            continue
+        r = measure_gpu(torch, mode, args.numel, args.steps, args.warmup, device)
+        also[mode] = {"params_per_s": r["params_per_s"], "ms_per_step": r["ms_per_step"], "step_ms_median": r["step_ms_median"],
+                      "kernel_ms": r["kernel_ms"], "kernel_ms_min": r["kernel_ms_min"], "kernel_ms_median": r["kernel_ms_median"],
+                      "kernel_ms_max": r["kernel_ms_max"], "bytes_per_param": r["bytes_per_param"], "achieved_gbs": r["achieved_gbs"],
+                      "frac_of_hbm_peak": r["achieved_gbs"] / HBM_PEAK_GBS,
+                      "frac_of_hbm_peak_through_adam_step": args.numel * r["bytes_per_param"] / r["ms_per_step"] / 1e6 / HBM_PEAK_GBS}
+    # steps of 0.5-1.5 ms: at least 100 of them, so that one slow step does not make the wall-clock figure
+    short_steps = max(args.steps, 100)
+    legs = [("grad_pass_fp16", lambda: measure_grad_pass(torch, args.numel, args.steps, args.warmup, device)),
+            ("ragged_4096_FULL_PRECISION", lambda: measure_ragged(torch, short_steps, args.warmup, device)),
+            ("ragged_4096_packed_views_FULL_PRECISION", lambda: measure_ragged(torch, short_steps, args.warmup, device, packed=True)),
+            ("ragged_4096_moving_gradients_FULL_PRECISION", lambda: measure_ragged(torch, short_steps, args.warmup, device, moving=True)),
+            ("c2_gpt2_small_148_tensors_MIXED_PRECISION", lambda: measure_c2(torch, short_steps, args.warmup, device)),
+            ("c5_llama7b_291_tensors_PURE_FP16", lambda: measure_c5(torch, min(args.steps, 10), min(args.warmup, 3), device))]
+    if not args.no_cpu:
+        legs.append(("c1_flat_2pow20_FULL_PRECISION_10_steps", lambda: measure_c1(torch, device)))
+    for key, leg in legs:
+        if wanted(key):
+            also[key] = leg()
     cpu = None if args.no_cpu else measure_cpu(torch, args.mode, args.cpu_numel)
 
     workload = f"flat_shard_{args.numel}_{args.mode}"

@@ -110,10 +110,10 @@ struct Options {
 int64_t default_lds_throttle(int mode, int64_t total_elems) {
     switch (mode) {
         case FSADAM_FULL_PRECISION:
-        case FSADAM_FULL_PRECISION_FP16_COPY: return total_elems < 20000000 ? 14080 : 15360;
-        case FSADAM_MIXED_PRECISION: return 15360;
-        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return total_elems < 50000000 ? 11520 : 12288;
-        default: return 12288;
+        case FSADAM_FULL_PRECISION_FP16_COPY:
+        case FSADAM_MIXED_PRECISION: return total_elems < 50000000 ? 14080 : 15360;
+        case FSADAM_MEMORY_EFFICIENT_MIXED_PRECISION: return total_elems < 500000000 ? 11520 : 12288;
+        default: return total_elems < 50000000 ? 11520 : 12288;
     }
 }
 Options g_opt;
@@ -1315,6 +1315,18 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
         return fail(FSADAM_EINVAL, "gradient list needs " + std::to_string(n_groups) + " workgroups, fsadam_grad_pass_noalloc holds partial results for at most " +
                                        std::to_string(FSADAM_NOALLOC_MAX_WORKGROUPS) + " (use fsadam_grad_pass)");
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    // every GPU has its own copy of the array: the one this call uses must be the one the stream runs on
+    if (stream) {
+        hipDevice_t stream_device = -1;
+        int current = -1;
+        FS_HIP(hipGetDevice(&current));
+        if (hipStreamGetDevice(stream, &stream_device) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(FSADAM_EINVAL, "the stream could not be asked for its device");
+        }
+        if ((int)stream_device != current)
+            return fail(FSADAM_EINVAL, "the stream belongs to device " + std::to_string((int)stream_device) + ", the current device is " + std::to_string(current));
+    }
     unsigned char* base = nullptr;
     if (int rc = scratch_on_current_device(&base)) return rc;
     ChunkDesc* table = reinterpret_cast<ChunkDesc*>(base);
