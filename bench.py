@@ -241,13 +241,21 @@ def measure_grad_pass(torch, numel, steps, warmup, device):
         for _ in range(warmup):
             grad_pass([g], inv, write_back=write_back)
         torch.cuda.synchronize()
+        # K passes between two events for the rate (a pass is three launches and takes 0.5-1 ms: an event behind every one
+        # would be part of what is timed), then K more with an event behind each for the spread
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            grad_pass([g], inv, write_back=write_back)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
         events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         events[0].record()
         for i in range(steps):
             grad_pass([g], inv, write_back=write_back)
             events[i + 1].record()
         torch.cuda.synchronize()
-        ms = events[0].elapsed_time(events[steps]) / steps
         median = spread([events[i].elapsed_time(events[i + 1]) for i in range(steps)])["median"]
         out[name] = {"ms": ms, "ms_median": median, "bytes_per_param": bpp, "achieved_gbs": numel * bpp / ms / 1e6,
                      "frac_of_hbm_peak": numel * bpp / ms / 1e6 / HBM_PEAK_GBS, "frac_at_median": numel * bpp / median / 1e6 / HBM_PEAK_GBS}
