@@ -17,7 +17,7 @@ MEMORY_EFFICIENT_MIXED_PRECISION = 2
 PURE_FP16 = 3
 FULL_PRECISION_FP16_COPY = 4
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libfsadam.so")
 

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define FSADAM_ABI_VERSION 3
+#define FSADAM_ABI_VERSION 4
 
 /* Precision modes = the four dtype combinations the reference dispatches on
  * (fairscale/clib/fused_adam_cuda/fused_adam_cuda_kernel.cu:172-256; Python enum
