@@ -115,8 +115,10 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
 
 /* Tuning knobs, by name; returns FSADAM_EINVAL for an unknown name or a value out of range.
  *   "lds_throttle"  bytes of untouched LDS given to every workgroup, which caps how many workgroups
- *                   share a compute unit (160 KiB / lds_throttle); 0 = no cap, -1 = the measured
- *                   per-mode default (12-15 KiB, default)
+ *                   share a compute unit (LDS is handed out in granules of 1280 bytes, 128 per compute unit:
+ *                   B bytes allow floor(128 / ceil(B / 1280)) workgroups); 0 = no cap, -1 (default) = chosen
+ *                   by precision mode and list size (11-15 KiB: 10 waves per compute unit in the 28-byte
+ *                   modes, 12 in the others, one step more for small lists)
  *   "merge_runs"    1 (default): consecutive rows of a list that continue each other in every stream (p, m, v, g and
  *                   the fp16 copy each start where the row before ended: parameters that are back-to-back views of
  *                   one buffer, with gradients and state laid out alike) are laid out as ONE tensor, so that a
@@ -134,9 +136,9 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   running on the caller's stream; 0: the copy is enqueued on the caller's stream
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
  *                   4 for one that writes the gradients back (default 0)
- *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 16384 / 12288 likewise
+ *   "grad_lds_throttle"  gradient pass: LDS ballast per workgroup in bytes; -1 = 14080 / 12800 likewise
  *   "grad_waves"    gradient pass: tiles (one wave each) per workgroup, 1, 4 or 16; the workgroup writes one
- *                   partial result.  0 = 16 for a read-only pass, 1 for one that writes back (default 0)
+ *                   partial result.  0 = 1 for either kind of pass (default 0)
  * A workgroup of the step is one wave64 handling one vector per lane and stream, tiles are taken in dispatch order
  * and full tiles of streams that are only element-aligned use the same vector instructions: the alternatives
  * (128/256 threads, two vectors per lane, an XCD-aware tile order, element-wise tiles, smaller shared chunks)
