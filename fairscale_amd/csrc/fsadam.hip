@@ -59,11 +59,11 @@
 // array per GPU, part of the loaded code object, held until the process ends.  Layout: the table
 // (FSADAM_NOALLOC_MAX_DESCRIPTORS rows of 64 bytes), then the partials of the tiles' workgroups
 // (FSADAM_NOALLOC_MAX_WORKGROUPS, and 7 more because the slots are handed out in eights), of the second reduction
-// stage (512) and the total (1), 16 bytes each.
+// stage (512) and the total (1), 16 bytes each, and 16 bytes that say which call owns the array (fsadam_put_descs).
 // In host code the name below is only a handle for hipGetSymbolAddress: the device address is looked up
 // once per device (scratch_on_current_device) and only that pointer is ever handed to a kernel.
 constexpr size_t kScratchTableBytes = (size_t)FSADAM_NOALLOC_MAX_DESCRIPTORS * 64;
-constexpr size_t kScratchPartials = (size_t)FSADAM_NOALLOC_MAX_WORKGROUPS + 7 + 512 + 1;  // 7: the slots are handed out in eights
+constexpr size_t kScratchPartials = (size_t)FSADAM_NOALLOC_MAX_WORKGROUPS + 7 + 512 + 1 + 1;  // 7: the slots are handed out in eights; the last 16 bytes: who owns the array
 constexpr size_t kScratchBytes = kScratchTableBytes + kScratchPartials * 16;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
@@ -879,7 +879,7 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
 template <typename T>
 int grad_launch(const ChunkDesc* table, const Layout& L, int64_t waves, int64_t items, size_t lds, float inv_scale, const float* inv_scale_dev,
                 int write_back, GradPartial* first, GradPartial* second, GradPartial* total, float* found_inf, double* sum_squares,
-                float* abs_max, hipStream_t stream) {
+                float* abs_max, hipStream_t stream, uint32_t* owner = nullptr, uint32_t ticket = 0) {
     const int64_t n_blocks = L.blocks();
     const TileMap map = tile_map(L);
     const int64_t n_groups = ceil_div(n_blocks, waves);
@@ -907,9 +907,9 @@ int grad_launch(const ChunkDesc* table, const Layout& L, int64_t waves, int64_t 
     const uint32_t blocks2 = (uint32_t)std::max<int64_t>(1, std::min<int64_t>(kReduceBlocks, ceil_div(n_slots, 1024)));
     const uint32_t per_block = (uint32_t)ceil_div(n_slots, blocks2);
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(blocks2), dim3(256), 0, stream, first, (uint32_t)n_slots, per_block, second, 0, 0,
-                       (float*)nullptr, (double*)nullptr, (float*)nullptr, per_xcd, (uint32_t)n_groups);
+                       (float*)nullptr, (double*)nullptr, (float*)nullptr, per_xcd, (uint32_t)n_groups, (uint32_t*)nullptr, 0u);
     hipLaunchKernelGGL(fsadam_grad_reduce, dim3(1), dim3(256), 0, stream, second, blocks2, blocks2, total, 1, (int)(sizeof(T) == 2),
-                       found_inf, sum_squares, abs_max, 0u, 0u);
+                       found_inf, sum_squares, abs_max, 0u, 0u, owner, ticket);
     FS_HIP(hipGetLastError());
     return FSADAM_OK;
 }
@@ -1336,20 +1336,28 @@ int fsadam_grad_pass_noalloc(const FsGradTensor* grads, int64_t n_tensors, int g
     if (!grad_fill_table(g_scratch_staging, L, grads, n_tensors, grad_elem_size(grad_dtype), 1))
         return fail(FSADAM_EINVAL, "internal error: descriptor count differs from the layout");
     // The table travels in kernel arguments, kDescsPerPut rows per launch: no copy engine, no staging buffer of
-    // the runtime's, nothing a capture could not record.
-    for (int64_t at = 0; at < n_descs; at += kDescsPerPut) {
+    // the runtime's, nothing a capture could not record.  The first of these launches (there is always one) takes
+    // possession of the array for this call, the last reduction gives it back: see fsadam_put_descs.
+    uint32_t* owner = reinterpret_cast<uint32_t*>(total + 1);
+    static uint32_t next_ticket = 0;  // guarded by g_scratch_mutex
+    if (++next_ticket == 0) ++next_ticket;
+    const uint32_t ticket = next_ticket;
+    int64_t at = 0;
+    do {
         const int64_t count = std::min<int64_t>(kDescsPerPut, n_descs - at);
         DescBatch batch;
         std::memcpy(batch.rows, g_scratch_staging + at, (size_t)count * sizeof(ChunkDesc));
-        hipLaunchKernelGGL(fsadam_put_descs, dim3(1), dim3(64), 0, stream, table, batch, (uint32_t)at, (uint32_t)count);
-    }
+        hipLaunchKernelGGL(fsadam_put_descs, dim3(1), dim3(64), 0, stream, table, batch, (uint32_t)at, (uint32_t)count, owner, ticket);
+        at += kDescsPerPut;
+    } while (at < n_descs);
     FS_HIP(hipGetLastError());
-    // Every partial a reduction reads was written by this call's tiles; nothing in the scratch has to start at zero.
+    // Every partial a reduction reads was written by this call's tiles; nothing in the scratch has to start at zero
+    // except the two words that say who owns it, which every call leaves at zero.
     return grad_dtype == FSADAM_GRAD_F16
                ? grad_launch<_Float16>(table, L, waves, items, lds, inv_scale, inv_scale_dev, write_back, first, second, total, found_inf_dev,
-                                       sum_squares_dev, abs_max_dev, stream)
+                                       sum_squares_dev, abs_max_dev, stream, owner, ticket)
                : grad_launch<float>(table, L, waves, items, lds, inv_scale, inv_scale_dev, write_back, first, second, total, found_inf_dev,
-                                    sum_squares_dev, abs_max_dev, stream);
+                                    sum_squares_dev, abs_max_dev, stream, owner, ticket);
 }
 
 int fsadam_clear_cache(void) {

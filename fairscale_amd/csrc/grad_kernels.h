@@ -247,7 +247,7 @@ __global__ __launch_bounds__(64 * WAVES) void fsadam_grad_tiles(const ChunkDesc*
 __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __restrict__ in, uint32_t n, uint32_t per_block,
                                                           GradPartial* __restrict__ out, int publish, int is_half,
                                                           float* found_inf, double* sum_squares, float* abs_max,
-                                                          uint32_t per_xcd, uint32_t n_groups) {
+                                                          uint32_t per_xcd, uint32_t n_groups, uint32_t* owner, uint32_t ticket) {
     __shared__ double s_sum[256];
     __shared__ uint32_t s_stored[256];
     __shared__ uint32_t s_incoming[256];
@@ -282,6 +282,24 @@ __global__ __launch_bounds__(256) void fsadam_grad_reduce(const GradPartial* __r
         out[blockIdx.x].incoming_max = s_incoming[0];
         return;
     }
+    if (owner) {
+        // The pass ran on memory that every call on this GPU shares (see fsadam_put_descs).  It is good only if this
+        // call still owns that memory and found it free when it began; otherwise another call's kernels ran in between
+        // and everything this pass computed is suspect: all three outputs become NaN (a flag that is not zero reads as
+        // an overflow to every caller, so the step is skipped rather than taken on a wrong norm).
+        const uint32_t holder = __hip_atomic_load(owner, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool spoiled = holder != ticket || owner[1] != 0u;
+        if (holder == ticket) {  // ours to give back
+            owner[1] = 0u;
+            __hip_atomic_store(owner, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (spoiled) {
+            if (found_inf) *found_inf = __builtin_nanf("");
+            if (sum_squares) *sum_squares = __builtin_nan("");
+            if (abs_max) *abs_max = __builtin_nanf("");
+            return;
+        }
+    }
     const uint32_t inf_pattern = is_half ? 0x7c00u : 0x7f800000u;
     if (s_incoming[0] >= inf_pattern && found_inf) *found_inf = 1.0f;  // set, never cleared: the caller zero-fills it
     if (sum_squares) *sum_squares = s_sum[0];
@@ -300,7 +318,17 @@ constexpr int kDescsPerPut = 48;
 struct DescBatch {
     ChunkDesc rows[kDescsPerPut];
 };
-__global__ __launch_bounds__(64) void fsadam_put_descs(ChunkDesc* __restrict__ table, DescBatch batch, uint32_t first, uint32_t count) {
+// The first launch of a call (first == 0) also takes possession of the memory the table and the partial results live in:
+// owner[0] holds the ticket of the call that is using it (0: free), owner[1] whether that call found it taken when it
+// began.  Calls that overlap on one GPU (two streams without an order between them, a replaying graph beside an eager
+// call) overwrite each other's table and partials; with the two words each of them finds out at its end (see
+// fsadam_grad_reduce) and reports NaN instead of a number that may be wrong.
+__global__ __launch_bounds__(64) void fsadam_put_descs(ChunkDesc* __restrict__ table, DescBatch batch, uint32_t first, uint32_t count,
+                                                        uint32_t* owner, uint32_t ticket) {
+    if (first == 0 && threadIdx.x == 0) {
+        const uint32_t before = __hip_atomic_exchange(owner, ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        owner[1] = before != 0u ? 1u : 0u;
+    }
     constexpr uint32_t kWords = sizeof(ChunkDesc) / sizeof(uint32_t);
     gptr<uint32_t> out = (gptr<uint32_t>)reinterpret_cast<uint32_t*>(table + first);
     const uint32_t* in = reinterpret_cast<const uint32_t*>(batch.rows);

@@ -260,13 +260,18 @@ int fsadam_grad_pass(const FsGradTensor* grads, int64_t n_tensors, int grad_dtyp
  * differently).  The call makes no hipMalloc / hipFree / hipHostMalloc, creates no stream or event and copies
  * nothing with the copy engines: the descriptor table travels in kernel arguments (one small launch per 48
  * rows) and lives, with the partial results, in an array that is part of the library's code object,
- * FSADAM_NOALLOC_MAX_DESCRIPTORS * 64 + (FSADAM_NOALLOC_MAX_WORKGROUPS + 520) * 16 bytes (1.26 MiB) per GPU,
+ * FSADAM_NOALLOC_MAX_DESCRIPTORS * 64 + (FSADAM_NOALLOC_MAX_WORKGROUPS + 521) * 16 bytes (1.26 MiB) per GPU,
  * held until the process ends.  A list that needs more descriptors or workgroups than that is refused with
  * FSADAM_EINVAL (a workgroup covers 65536 fp16 / 32768 fp32 elements when the pass only reads, half as many
  * when it writes back: at least 1.07e9 elements in every case; a tensor of 131072 elements or more takes one
  * descriptor per 2^16..2^24 elements, smaller ones up to 16, plus one for a misaligned start).  Tuning options
  * are not consulted.  All calls on one GPU share that GPU's array: calls whose kernels may overlap (different
- * streams without an order between them, or two threads) race; calls on one stream are ordered by it.  The call may
+ * streams without an order between them, a replaying graph beside an eager call) race; calls on one stream are ordered
+ * by it.  The race is not prevented but it is noticed: the first kernel of a call takes possession of the array and the
+ * last gives it back, and a call that did not own the array from its beginning to its end reports NaN in all three
+ * outputs (a flag that is not zero reads as an overflow, so the step is skipped) instead of numbers that may be wrong;
+ * the gradients of a pass that writes back are then undefined.  Lists that overlap in time must be such that either
+ * call's kernels may read the other's descriptors; the stream must belong to the current device.  The call may
  * be recorded into a HIP graph (its scalars do not depend on a step count); make the first call on a device outside
  * any capture, since that call looks up the array's address. */
 #define FSADAM_NOALLOC_MAX_DESCRIPTORS 4096

@@ -140,6 +140,49 @@ def test_a_shard_sized_buffer_then_a_small_one(cuda_device):
     _compare([1000], torch.float16, 1.0 / 1024, False, cuda_device, seed=8)
 
 
+def test_calls_that_overlap_report_nan_or_the_right_numbers(cuda_device):
+    """Calls on two streams without an order between them share the GPU's one array; the library cannot prevent that,
+    but each call finds out at its end whether it owned the array from beginning to end, and reports NaN in all three
+    outputs if it did not.  Here both streams pass the SAME list (so whatever mixture of the two tables a kernel reads
+    stays inside the tensors) and nothing is written back; every result must be either all NaN or exactly the result of
+    the call made alone, and a call made alone afterwards must be right again (the array was given back)."""
+    from fairscale_amd import _cabi
+
+    L = _cabi.lib()
+    gen = torch.Generator(device="cpu").manual_seed(21)
+    grads = [(torch.randn(n, generator=gen) * 0.05).half().to(cuda_device) for n in (3_000_001, 70_001, 9)]
+    grads.append(torch.zeros(60_000_000, dtype=torch.float16, device=cuda_device).normal_(0, 0.05))
+    rows = _rows(grads)
+    alone = _call("fsadam_grad_pass_noalloc", grads, 0.25, False)
+    assert not np.isnan(alone[1]) and alone[0] == 0.0
+    streams = [torch.cuda.Stream(cuda_device), torch.cuda.Stream(cuda_device)]
+    outs = [[torch.zeros(1, device=cuda_device), torch.zeros(1, device=cuda_device, dtype=torch.float64), torch.zeros(1, device=cuda_device)]
+            for _ in streams]
+    spoiled = 0
+    for rnd in range(8):
+        print(f"[noalloc] overlap round {rnd}", flush=True)
+        torch.cuda.synchronize(cuda_device)
+        for flag, _, _ in outs:
+            flag.zero_()
+        torch.cuda.synchronize(cuda_device)
+        for k in ((0, 1) if rnd % 2 == 0 else (1, 0)):
+            flag, ssq, amax = outs[k]
+            _cabi.check(L.fsadam_grad_pass_noalloc(rows, len(grads), _cabi.GRAD_F16, 0.25, None, 0, flag.data_ptr(), ssq.data_ptr(),
+                                                   amax.data_ptr(), streams[k].cuda_stream))
+        torch.cuda.synchronize(cuda_device)
+        for flag, ssq, amax in outs:
+            got = (flag.item(), ssq.item(), amax.item())
+            if all(np.isnan(x) for x in got):
+                spoiled += 1
+            else:
+                assert got == alone, f"round {rnd}: a call that overlapped another reported {got}, alone it reports {alone}"
+    print(f"[noalloc] {spoiled} of 16 overlapping calls reported NaN", flush=True)
+    again = _call("fsadam_grad_pass_noalloc", grads, 0.25, False)
+    if any(np.isnan(x) for x in again):  # at most the first call behind a spoiled pair may still find the array taken
+        again = _call("fsadam_grad_pass_noalloc", grads, 0.25, False)
+    assert again == alone
+
+
 def test_lists_beyond_the_scratch_are_refused(cuda_device):
     from fairscale_amd import _cabi
 
