@@ -764,7 +764,8 @@ def main():
         "config": {"workload": workload, "numel": args.numel, "precision": args.mode, "tensors": 1,
                    "storage": {"FULL_PRECISION": "p,g,m,v fp32", "MIXED_PRECISION": "p,m,v fp32; g, copy-out fp16",
                                "MEMORY_EFFICIENT_MIXED_PRECISION": "p,g fp16; m,v fp32", "PURE_FP16": "p,g,m,v fp16"}[args.mode], "grad_scale": 1024.0 if args.mode != "FULL_PRECISION" else 1.0,
-                   "entry": "fairscale_amd.optim.Adam.step", **main_res["plan"],
+                   "entry": "fairscale_amd.optim.Adam.step", "library": os.path.relpath(_cabi.library_path(), REPO), "abi": _cabi.ABI_VERSION,
+                   **main_res["plan"],
                    "options": {k: _cabi.get_option(k) for k in ("lds_throttle", "merge_runs", "align_heads", "mid_tiles")}},
         "roofline": {"bound": "hbm", "achieved": main_res["achieved_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": main_res["achieved_gbs"] / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
