@@ -56,3 +56,18 @@ def test_benchmark_configurations_have_the_sizes_the_baseline_names():
     assert "124_439_808" in src and "6_738_415_616" in src and "== 148" in src and "== 291" in src
     assert sum(C.numel(s) for s in C.gpt2_small_shapes()) == 124_439_808 and len(C.gpt2_small_shapes()) == 148
     assert sum(C.numel(s) for s in C.llama7b_shapes()) == 6_738_415_616 and len(C.llama7b_shapes()) == 291
+
+
+def test_measurement_selectors_are_options_of_the_benchmark(monkeypatch):
+    """--also-only picks secondary measurements by the start of their key, --lds-sweep takes a list of ballasts; both are
+    what the commands in profiles/ use, so they must stay spelled this way."""
+    import bench
+
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--also-only", "grad_pass", "--also-only", "c5_", "--lds-sweep", "8960,12288", "--steps", "3"])
+    args = bench.parse_args()
+    assert args.also_only == ["grad_pass", "c5_"] and args.lds_sweep == "8960,12288" and args.steps == 3
+    for name in os.listdir(os.path.join(REPO, "profiles")):
+        text = open(os.path.join(REPO, "profiles", name)).read()
+        for flag in ("--also-only", "--lds-sweep", "--micro", "--calib-copy-bytes", "--no-also", "--no-cpu"):
+            if flag in text:
+                assert flag in open(os.path.join(REPO, "bench.py")).read(), f"profiles/{name} uses {flag}, which bench.py no longer has"
