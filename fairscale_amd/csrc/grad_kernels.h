@@ -318,14 +318,14 @@ constexpr int kDescsPerPut = 48;
 struct DescBatch {
     ChunkDesc rows[kDescsPerPut];
 };
-// The first launch of a call (first == 0) also takes possession of the memory the table and the partial results live in:
+// With `owner` set, the first launch of a call (first == 0) also takes possession of the memory the table and the partial results live in:
 // owner[0] holds the ticket of the call that is using it (0: free), owner[1] whether that call found it taken when it
 // began.  Calls that overlap on one GPU (two streams without an order between them, a replaying graph beside an eager
 // call) overwrite each other's table and partials; with the two words each of them finds out at its end (see
 // fsadam_grad_reduce) and reports NaN instead of a number that may be wrong.
 __global__ __launch_bounds__(64) void fsadam_put_descs(ChunkDesc* __restrict__ table, DescBatch batch, uint32_t first, uint32_t count,
                                                         uint32_t* owner, uint32_t ticket) {
-    if (first == 0 && threadIdx.x == 0) {
+    if (owner && first == 0 && threadIdx.x == 0) {
         const uint32_t before = __hip_atomic_exchange(owner, ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         owner[1] = before != 0u ? 1u : 0u;
     }
