@@ -131,7 +131,8 @@ float fsadam_step_size(float lr, float beta1, float beta2, int step, int bias_co
  *                   under 131072 elements): 0 (every such tile has its own descriptor) or a power of two up to 64
  *                   (default 16).  Shared descriptors make the table of a many-tensor list 10x shorter, which is
  *                   what is sent again when a pointer of the list moves
- *   "upload_stream" 1 (default): a new descriptor table is copied to the device on a stream the library owns,
+ *   "upload_stream" (tables of more than 48 rows; a shorter one travels in the arguments of one small launch on the
+ *                   caller's stream)  1 (default): a new descriptor table is copied to the device on a stream the library owns,
  *                   and the caller's stream waits for that copy's event, so the copy overlaps the step still
  *                   running on the caller's stream; 0: the copy is enqueued on the caller's stream
  *   "grad_items"    gradient pass: 16-byte vectors per lane, 2, 4 or 8; 0 = 8 for a read-only pass,
