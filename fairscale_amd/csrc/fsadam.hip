@@ -40,6 +40,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -372,7 +373,8 @@ struct UseMark {
 struct TableSlot {
     int64_t cap_descs = 0;
     ChunkDesc* d_table = nullptr;
-    ChunkDesc* h_table = nullptr;  // pinned
+    ChunkDesc* h_table = nullptr;  // pinned, or ordinary host memory for a table short enough to travel in kernel arguments
+    bool pinned = false;
     UseMark mark;
     hipEvent_t uploaded = nullptr;  // the copy of h_table into d_table, when it went over the library's own stream
 };
@@ -481,10 +483,41 @@ void upload_stream_destroy(hipStream_t* own) {
 void slot_release(TableSlot& slot) {
     (void)mark_wait(slot.mark);
     if (slot.d_table) (void)hipFree(slot.d_table);
-    if (slot.h_table) (void)hipHostFree(slot.h_table);
+    if (slot.h_table) {
+        if (slot.pinned) (void)hipHostFree(slot.h_table);
+        else std::free(slot.h_table);
+    }
     slot.d_table = slot.h_table = nullptr;
     slot.cap_descs = 0;
+    slot.pinned = false;
     slot.mark.used = slot.mark.pending = false;
+}
+
+// Room for a table of n_descs rows in a slot nothing reads any more.  A table short enough to travel in kernel arguments
+// (upload_table) is staged in ordinary host memory: pinning a page costs 35-140 us, which is most of what the first
+// steps of a small list would spend.
+int slot_reserve(TableSlot& slot, int64_t n_descs) {
+    const bool want_pinned = n_descs > kDescsPerPut;
+    if (n_descs <= slot.cap_descs && (slot.pinned || !want_pinned)) return FSADAM_OK;
+    slot_release(slot);
+    const int64_t cap = want_pinned ? std::max<int64_t>(n_descs + n_descs / 8, 64) : kDescsPerPut;
+    if (hipMalloc(reinterpret_cast<void**>(&slot.d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
+        slot.d_table = nullptr;
+        return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
+    }
+    if (want_pinned) {
+        if (hipHostMalloc(reinterpret_cast<void**>(&slot.h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) slot.h_table = nullptr;
+    } else {
+        slot.h_table = static_cast<ChunkDesc*>(std::malloc((size_t)cap * sizeof(ChunkDesc)));
+    }
+    if (!slot.h_table) {
+        (void)hipFree(slot.d_table);
+        slot.d_table = nullptr;
+        return fail(FSADAM_ENOMEM, "allocation of the descriptor staging buffer failed");
+    }
+    slot.pinned = want_pinned;
+    slot.cap_descs = cap;
+    return FSADAM_OK;
 }
 
 // The scalars of a step (step size, scales) travel by value in the kernel arguments and the table slots
@@ -588,20 +621,8 @@ int plan_set_tensors(FsAdamPlan* plan, const FsAdamTensor* tensors, int64_t n, h
     if (rc) return rc;
     rc = mark_wait(slot.mark);
     if (rc) return rc;
-    if (n_descs > slot.cap_descs) {
-        slot_release(slot);
-        const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
-        if (hipMalloc(reinterpret_cast<void**>(&slot.d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
-            slot.d_table = nullptr;
-            return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
-        }
-        if (hipHostMalloc(reinterpret_cast<void**>(&slot.h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
-            (void)hipFree(slot.d_table);
-            slot.d_table = slot.h_table = nullptr;
-            return fail(FSADAM_ENOMEM, "hipHostMalloc of the descriptor staging buffer failed");
-        }
-        slot.cap_descs = cap;
-    }
+    rc = slot_reserve(slot, n_descs);
+    if (rc) return rc;
     // descriptors of large tensors first, then the middle-sized ones, then one per tile: one launch covers all
     ChunkDesc* large = slot.h_table;
     ChunkDesc* mid = large + L.n_large_descs;
@@ -839,20 +860,8 @@ int grad_plan_set(GradPlan* plan, const FsGradTensor* grads, int64_t n, hipStrea
     if (rc) return rc;
     rc = mark_wait(slot.mark);
     if (rc) return rc;
-    if (n_descs > slot.cap_descs) {
-        slot_release(slot);
-        const int64_t cap = std::max<int64_t>(n_descs + n_descs / 8, 64);
-        if (hipMalloc(reinterpret_cast<void**>(&slot.d_table), cap * sizeof(ChunkDesc)) != hipSuccess) {
-            slot.d_table = nullptr;
-            return fail(FSADAM_ENOMEM, "hipMalloc of the descriptor table failed");
-        }
-        if (hipHostMalloc(reinterpret_cast<void**>(&slot.h_table), cap * sizeof(ChunkDesc), hipHostMallocDefault) != hipSuccess) {
-            (void)hipFree(slot.d_table);
-            slot.d_table = slot.h_table = nullptr;
-            return fail(FSADAM_ENOMEM, "hipHostMalloc of the descriptor staging buffer failed");
-        }
-        slot.cap_descs = cap;
-    }
+    rc = slot_reserve(slot, n_descs);
+    if (rc) return rc;
     if (n_blocks + kSlotSlack + kReduceBlocks + 1 > plan->cap_partials) {
         // the partials may still be read by the reduction of the previous call
         rc = mark_wait(plan->partials_mark);
